@@ -1,0 +1,230 @@
+/*
+ * kvcm_hip.h -- C-ABI of libkvcm_hip.so: the MI355X (gfx950) save/load hot path of the
+ * Tair KVCache Manager connector.
+ *
+ * Two families of entry points:
+ *   - block-key hashing of token-ID sequences (the manager's GenKeyVector / hashInt64Array and its
+ *     siblings), batched over requests;
+ *   - gather/scatter of paged KV blocks between an engine's per-layer paged cache ("pool") and the
+ *     contiguous block-major staging buffers that the storage SDKs read and write.
+ *
+ * Conventions
+ *   - every pointer whose name starts with d_ is DEVICE memory, readable/writable by kernels on the
+ *     current HIP device; everything else is host memory;
+ *   - all entry points are asynchronous on `stream` (a hipStream_t passed as void*; NULL = null stream),
+ *     never synchronise, never allocate, never switch device, and keep no global mutable state, so they
+ *     can be called concurrently from many host threads (the reference calls its kernels from a
+ *     32-thread pool: kv_cache_manager/py_connector/vllm/data_transfer.py:80-93);
+ *   - device buffers passed in must stay alive until `stream` has executed the call;
+ *   - return value: 0 = OK, negative = KVCM_ERR_* (argument rejected, nothing launched),
+ *     positive = a hipError_t reported by the launch.
+ *
+ * Every prototype cites the reference interface it replaces (paths relative to the reference root).
+ */
+#ifndef KVCM_HIP_H
+#define KVCM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *kvcm_stream_t;
+
+#define KVCM_OK 0
+#define KVCM_ERR_INVALID_ARG (-1) /* null pointer, non-positive size, inconsistent shape */
+#define KVCM_ERR_ALIGNMENT (-2)   /* an address or stride is not aligned as the entry point requires */
+#define KVCM_ERR_TOO_LARGE (-3)   /* a size exceeds what the launch geometry can express */
+
+/* Library version: major*10000 + minor*100 + patch. */
+int32_t kvcm_hip_version(void);
+
+/* Text for a return code of this library (negative codes) or of HIP (positive codes). */
+const char *kvcm_hip_error_string(int32_t code);
+
+/* ------------------------------------------------------------------------------------------------
+ * Block-key hashing
+ * ------------------------------------------------------------------------------------------------ */
+
+/*
+ * Parent-chained block keys of R token sequences in one launch.
+ * Replaces: GenKeyVector(tokens, block_size)  kv_cache_manager/manager/cache_manager.cc:76-87
+ *           over hashInt64Array / hashInt64Func kv_cache_manager/manager/hash_util.h:8-24
+ * (one call per request in the reference; here R requests per launch).
+ *
+ * Request r owns tokens d_tokens[d_token_offsets[r] .. d_token_offsets[r+1]) and produces
+ * n_r = len_r / block_size keys (floor; a trailing partial block yields no key), written to
+ * d_keys[d_key_offsets[r] .. d_key_offsets[r] + n_r). Key i is the running 64-bit state, started at
+ * `seed` (the reference uses 0), after folding tokens [0, (i+1)*block_size) with
+ *   h <- h XOR (v + 0x9e3779b97f4a7c15 + (h << 12) + (h >> 32))   (int64, arithmetic >>, mod 2^64).
+ * d_key_offsets may be NULL when every request has the same length L = token_offsets[1]-[0]; keys of
+ * request r then start at r * (L / block_size).
+ */
+int32_t kvcm_hip_hash_tokens(const int64_t *d_tokens, const int64_t *d_token_offsets, int32_t R,
+                             int32_t block_size, int64_t seed, int64_t *d_keys,
+                             const int64_t *d_key_offsets, kvcm_stream_t stream);
+
+/* Same function for int32 token IDs (sign-extended to int64 before hashing): engines hold token IDs as
+ * int32, the wire format widens them (kv_cache_manager/protocol/protobuf/meta_service.proto:199). */
+int32_t kvcm_hip_hash_tokens_i32(const int32_t *d_tokens, const int64_t *d_token_offsets, int32_t R,
+                                 int32_t block_size, int64_t seed, int64_t *d_keys,
+                                 const int64_t *d_key_offsets, kvcm_stream_t stream);
+
+/*
+ * Prefix-chained keys from per-block digests: keys[i] = fold of digests[0..i].
+ * Replaces: ApplyPrefixHash  kv_cache_manager/optimizer/trace_converter/trace_util.cc:47-56.
+ * Sequence r owns d_digests[d_offsets[r] .. d_offsets[r+1]) and writes the same index range of d_keys.
+ */
+int32_t kvcm_hip_prefix_chain(const int64_t *d_digests, const int64_t *d_offsets, int32_t R,
+                              int64_t *d_keys, kvcm_stream_t stream);
+
+/*
+ * int64 keys from strings: big-endian signed value of the first 8 bytes of SHA-256(bytes).
+ * Replaces: HiCacheKVCM._sha256_to_int64 / _prepare_block_keys
+ *           kv_cache_manager/py_connector/sglang/connector.py:397-415.
+ * String i is d_bytes[d_offsets[i] .. d_offsets[i+1]) (already UTF-8 encoded).
+ */
+int32_t kvcm_hip_sha256_first8_be(const uint8_t *d_bytes, const int64_t *d_offsets, int32_t N,
+                                  int64_t *d_out, kvcm_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Paged-KV gather / scatter
+ * ------------------------------------------------------------------------------------------------
+ * Pool: P separate arrays ("one per layer and K/V"), array p = rows of `row_bytes` bytes, row s at
+ *       d_ptr_table[p] + s * row_bytes (s = token slot). Order of p: layer-major, K before V
+ *       (kv_cache_manager/py_connector/vllm/v1_connector.py:405-413).
+ * Staging: slots of staging_block_stride_bytes; slot k holds one block as [P][T][row_bytes]
+ *       (kv_cache_manager/py_connector/kernel/batch_gather_scatter_helper.py:104), the exact bytes the
+ *       storage SDKs put at file offset blkid * location_spec_size.
+ * Work block b (b < B) names T token slots and one staging slot d_staging_idx[b]
+ * (NULL = slot b). Staging slots not named are left untouched; so are pool rows not named.
+ * Scatter with two work blocks that name the same pool row is a data race: callers must not do that.
+ * Data are moved as raw bytes; the element type never matters.
+ */
+
+/*
+ * gather:  staging[sb[b]][p][t][:] <- pool_p[idx[b][t]][:]      for all b < B, p < P, t < T
+ * Replaces: batch_gather_kv_caches + kv_cache_batch_gather_kernel
+ *           kv_cache_manager/py_connector/kernel/batch_gather_scatter_helper.py:33-136.
+ * d_token_idx is int32 [B][T] (token slot numbers), as the reference uploads it (:118).
+ * max_workgroups <= 0 fills the device; a positive value caps the grid (the reference's sm_count, :110).
+ */
+int32_t kvcm_hip_batch_gather(const void *const *d_ptr_table, int32_t P, void *d_staging,
+                              int64_t staging_block_stride_bytes, const int32_t *d_token_idx,
+                              const int32_t *d_staging_idx, int32_t B, int32_t T, int64_t row_bytes,
+                              int32_t max_workgroups, kvcm_stream_t stream);
+
+/*
+ * scatter: pool_p[idx[b][t]][:] <- staging[sb[b]][p][t][:]
+ * Replaces: batch_scatter_kv_caches + kv_cache_batch_scatter_kernel
+ *           kv_cache_manager/py_connector/kernel/batch_gather_scatter_helper.py:139-248.
+ */
+int32_t kvcm_hip_batch_scatter(const void *const *d_ptr_table, int32_t P, const void *d_staging,
+                               int64_t staging_block_stride_bytes, const int32_t *d_token_idx,
+                               const int32_t *d_staging_idx, int32_t B, int32_t T, int64_t row_bytes,
+                               int32_t max_workgroups, kvcm_stream_t stream);
+
+/*
+ * Block-table fast path: the T tokens of work block b are T / run_tokens runs of `run_tokens`
+ * consecutive slots; d_run_start is int32 [B][T / run_tokens] and holds the first slot of every run
+ * (engine_block_id * engine_block_size + offset). Equal to kvcm_hip_batch_gather on the expanded
+ * per-token index that generate_blocks_idx builds
+ * (kv_cache_manager/py_connector/vllm/v1_connector.py:308-320), without building it.
+ */
+int32_t kvcm_hip_paged_gather(const void *const *d_ptr_table, int32_t P, void *d_staging,
+                              int64_t staging_block_stride_bytes, const int32_t *d_run_start,
+                              int32_t run_tokens, const int32_t *d_staging_idx, int32_t B, int32_t T,
+                              int64_t row_bytes, int32_t max_workgroups, kvcm_stream_t stream);
+
+int32_t kvcm_hip_paged_scatter(const void *const *d_ptr_table, int32_t P, const void *d_staging,
+                               int64_t staging_block_stride_bytes, const int32_t *d_run_start,
+                               int32_t run_tokens, const int32_t *d_staging_idx, int32_t B, int32_t T,
+                               int64_t row_bytes, int32_t max_workgroups, kvcm_stream_t stream);
+
+/*
+ * General form behind all gather/scatter entry points.
+ *
+ *  - pool array p lives at d_ptr_table[p / ptrs_per_entry] + (p % ptrs_per_entry) * entry_stride_bytes:
+ *    ptrs_per_entry = 1 for a table of P pointers; ptrs_per_entry = 2 with entry_stride_bytes =
+ *    total_slots * row_bytes for one [2, total_slots, H] tensor per layer, K then V
+ *    (legacy layout, kv_cache_manager/py_connector/kernel/gather_scatter_helper.py:91-97);
+ *  - slot_limit > 0: runs whose first slot is >= slot_limit are skipped in both directions
+ *    (gather_scatter_helper.py:37-38,88-89); 0 = no limit;
+ *  - staging_tile_stride_bytes: distance between tile p and tile p+1 inside a staging slot;
+ *    T * row_bytes + trailer_bytes for the packed record;
+ *  - trailer: trailer_bytes > 0 appends to every (b, p) tile the bytes
+ *    d_trailer_ptr_table[p][d_trailer_idx[b] * trailer_bytes ..] (per-block quantisation scales of an
+ *    fp8 cache); on scatter they are written back. No counterpart in the reference, which has only the
+ *    one-pointer-per-layer MLA branch (kv_cache_manager/py_connector/vllm/v1_connector.py:398-403).
+ */
+typedef struct kvcm_copy_desc {
+    const void *const *d_ptr_table;
+    int32_t P;
+    int32_t ptrs_per_entry;
+    int64_t entry_stride_bytes;
+    void *d_staging;
+    int64_t staging_block_stride_bytes;
+    int64_t staging_tile_stride_bytes;
+    const int32_t *d_run_start;
+    const int32_t *d_staging_idx;
+    int32_t B;
+    int32_t T;
+    int32_t run_tokens;
+    int32_t slot_limit;
+    int64_t row_bytes;
+    const void *const *d_trailer_ptr_table;
+    const int32_t *d_trailer_idx;
+    int32_t trailer_bytes;
+    int32_t max_workgroups;
+} kvcm_copy_desc;
+
+int32_t kvcm_hip_gather_ex(const kvcm_copy_desc *desc, kvcm_stream_t stream);
+int32_t kvcm_hip_scatter_ex(const kvcm_copy_desc *desc, kvcm_stream_t stream);
+
+/*
+ * Token-slot indices of manager blocks on device:
+ *   out[b][i] = block_ids[(m_b*T_mgr + i) / T_eng] * T_eng + (m_b*T_mgr + i) % T_eng,  i < T_mgr
+ * Replaces: TairKvCacheConnector.generate_blocks_idx
+ *           kv_cache_manager/py_connector/vllm/v1_connector.py:308-320 (a Python double loop).
+ * n_local = length of d_local_block_ids; a token that falls beyond it (the reference asserts) makes
+ * the kernel write -1 for that entry and raise *d_error_flag (int32, may be NULL) to 1.
+ */
+int32_t kvcm_hip_generate_blocks_idx(const int32_t *d_manager_block_idxes, int32_t B,
+                                     const int32_t *d_local_block_ids, int32_t n_local, int32_t T_mgr,
+                                     int32_t T_eng, int32_t *d_out, int32_t *d_error_flag,
+                                     kvcm_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Buffer check (debug aid of the transfer client)
+ * ------------------------------------------------------------------------------------------------ */
+
+typedef struct kvcm_iov_device {
+    const void *base;
+    size_t size;
+} kvcm_iov_device;
+
+/*
+ * Per iov: reflected CRC-32 (poly 0xEDB88320, init 0xFFFFFFFF, final NOT) over the first cal_bytes and
+ * then the last cal_bytes bytes of the iov, one running CRC.
+ * Replaces: GetIovsCrcDevice  kv_cache_manager/client/src/internal/sdk/sdk_buffer_check_util.cu:21-44
+ * (the caller picks cal_bytes = min(KVCM_CHECK_IOV_BYTE_SIZE, iovs[0].size / 2) and skips the launch
+ * when it is 0, as sdk_buffer_check_util.cu:50-55 does).
+ */
+int32_t kvcm_hip_iov_crc32(const kvcm_iov_device *d_iovs, int32_t n, uint32_t *d_crc,
+                           size_t cal_bytes, kvcm_stream_t stream);
+
+/*
+ * Host helper, no device work: per block, the hashInt64 chain (seed 0) over the block's
+ * `iovs_per_block` CRCs, each zero-extended to 64 bits.
+ * Replaces: the loop at kv_cache_manager/client/src/internal/sdk/sdk_buffer_check_util.cc:56-60 over
+ * HashUtil::HashIntArray<uint32_t>  kv_cache_manager/common/hash_util.h:17-25.
+ */
+int32_t kvcm_blocks_hash_from_crcs(const uint32_t *crcs, int64_t n_crcs, int32_t iovs_per_block,
+                                   int64_t *out_hashes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KVCM_HIP_H */

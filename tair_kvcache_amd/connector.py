@@ -1,0 +1,239 @@
+"""The callers on either side of the gather/scatter kernels, as the vLLM connector arranges them.
+
+    generate_blocks_idx   TairKvCacheConnector.generate_blocks_idx  kv_cache_manager/py_connector/vllm/v1_connector.py:308-320
+    register_kv_caches    TairKvCacheConnector.register_kv_caches   kv_cache_manager/py_connector/vllm/v1_connector.py:360-445
+    MultiResult           kv_cache_manager/py_connector/vllm/data_transfer.py:18-36
+    DataTransferManager   kv_cache_manager/py_connector/vllm/data_transfer.py:39-244 (save_task :190-244, load_task :108-158)
+
+What is not here: the engine plugin classes, the HTTP manager client and the ZMQ coordinator (control plane).
+The transfer client is whatever object offers SaveKvCaches(uris, buffers) -> (code, uris) and
+LoadKvCaches(uris, buffers) -> code (kv_cache_manager/client/include/transfer_client.h:19-21).
+"""
+import math
+import threading
+from concurrent.futures import ThreadPoolExecutor
+from dataclasses import dataclass
+from typing import Any, Callable, Dict, List, Optional, Sequence
+
+import torch
+
+from . import _lib, client_types
+from ._torch_util import as_device_i32, lib, ptr, stream_handle
+from .kernel import batch_gather_scatter_helper
+from .kernel.gather_scatter_helper import CopyBufferAllocator
+
+
+def generate_blocks_idx(manager_block_idxes: Sequence[int], local_block_ids: Sequence[int],
+                        manager_block_size: int, local_block_size: int, device="cuda") -> torch.Tensor:
+    """int32 device tensor [B, manager_block_size]:
+    out[b][i] = local_block_ids[tok // local_block_size] * local_block_size + tok % local_block_size with
+    tok = manager_block_idxes[b] * manager_block_size + i. The reference builds this as nested Python lists;
+    here it is one kernel and the result never visits the host. Raises AssertionError, as the reference's
+    assert does, when a manager block reaches beyond local_block_ids."""
+    T_mgr, T_eng = int(manager_block_size), int(local_block_size)
+    B = len(manager_block_idxes)
+    out = torch.empty((B, T_mgr), dtype=torch.int32, device=device)
+    if B == 0:
+        return out
+    hi = max(manager_block_idxes) if not isinstance(manager_block_idxes, torch.Tensor) else int(
+        manager_block_idxes.max().item())
+    lo = min(manager_block_idxes) if not isinstance(manager_block_idxes, torch.Tensor) else int(
+        manager_block_idxes.min().item())
+    if lo < 0 or (hi * T_mgr + T_mgr - 1) // T_eng >= len(local_block_ids):
+        raise AssertionError("manager block reaches beyond local_block_ids")
+    m = as_device_i32(manager_block_idxes, out.device, "manager_block_idxes")
+    l = as_device_i32(local_block_ids, out.device, "local_block_ids")
+    rc = lib().kvcm_hip_generate_blocks_idx(ptr(m), B, ptr(l), l.numel(), T_mgr, T_eng, ptr(out), None,
+                                            stream_handle(out.device))
+    _lib.check(rc, "kvcm_hip_generate_blocks_idx")
+    return out
+
+
+def generate_run_starts(manager_block_idxes: Sequence[int], local_block_ids: Sequence[int],
+                        manager_block_size: int, local_block_size: int, device="cuda"):
+    """Block-table form of generate_blocks_idx: (run_start [B, manager_block_size // g], g) with
+    g = gcd(manager_block_size, local_block_size). A run of g tokens that starts at a multiple of g never
+    crosses an engine block, so run_start[b][j] = generate_blocks_idx(...)[b][j * g] describes the same rows."""
+    T_mgr, T_eng = int(manager_block_size), int(local_block_size)
+    g = math.gcd(T_mgr, T_eng)
+    groups = generate_blocks_idx(manager_block_idxes, local_block_ids, T_mgr // g, T_eng // g, device)
+    return groups * g, g
+
+
+@dataclass
+class KVCacheInfo:
+    """What register_kv_caches derives from the engine's cache tensors (kv_cache_manager/py_connector/common/types.py)."""
+    tp_rank: int
+    tp_size: int
+    kv_caches: Dict[str, torch.Tensor]
+    kvcache_ptr_tensor_cpu: torch.Tensor
+    kvcache_ptr_tensor_gpu: torch.Tensor
+    all_kvcache_ptr_tensor_gpu: torch.Tensor
+    layer_num: int
+    local_token_num: int
+    per_manager_location_spec_shape: tuple
+    per_manager_location_spec_byte_size: int
+    per_token_per_layer_dim_size: int
+    device: torch.device
+    dtype: torch.dtype
+
+
+def register_kv_caches(kv_caches: Dict[str, torch.Tensor], manager_block_size: int, local_block_size: int,
+                       use_mla: bool = False, tp_rank: int = 0, tp_size: int = 1) -> KVCacheInfo:
+    """Pointer tables and staging geometry for per-layer caches [2, block_num, block_size, kv_heads, head_dim]
+    (MLA: [block_num, block_size, latent_dim], one pointer per layer).
+
+    Order of the pointer table: layer-major, K before V (v1_connector.py:405-413); staging slot shape
+    [layers, 2, manager_block_size, kv_heads * head_dim] (:376-388) whose byte size is the location-spec size
+    the manager and the storage backends use as the per-block file stride."""
+    if len(kv_caches) == 0:
+        raise ValueError("kv_caches is empty")
+    first = next(iter(kv_caches.values()))
+    kv_dim = 1 if use_mla else 2
+    tok_axis = 1 if use_mla else 2
+    assert local_block_size == first.shape[tok_axis], "kv cache shape error"
+    for t in kv_caches.values():
+        assert t.is_contiguous(), "kv cache must be contiguous"
+        assert t.shape == first.shape and t.dtype == first.dtype, "kv cache shape error"
+    block_num = first.shape[tok_axis - 1]
+    dim = math.prod(first.shape[tok_axis + 1:])
+    itemsize = first.element_size()
+    layer_shape = [kv_dim, manager_block_size, dim]
+    row = first[0] if use_mla else first[0][0]  # [block_size, ...] of the first block
+    assert dim * itemsize == row[1].data_ptr() - row[0].data_ptr(), "kv cache shape error"
+    spec_shape = [len(kv_caches)] + layer_shape
+    spec_bytes = math.prod(spec_shape) * itemsize
+    names = list(kv_caches)
+    ptr_cpu = torch.tensor([kv_caches[n].data_ptr() for n in names], dtype=torch.int64)
+    if use_mla:
+        all_ptrs = [kv_caches[n].data_ptr() for n in names]
+    else:
+        all_ptrs = []
+        for n in names:
+            all_ptrs.append(kv_caches[n][0].data_ptr())
+            all_ptrs.append(kv_caches[n][1].data_ptr())
+    device = first.device
+    return KVCacheInfo(tp_rank, tp_size, kv_caches, ptr_cpu, ptr_cpu.to(device),
+                       torch.tensor(all_ptrs, dtype=torch.int64).to(device), len(kv_caches),
+                       block_num * local_block_size, tuple(spec_shape), spec_bytes, dim, device, first.dtype)
+
+
+class MultiResult:
+    """Collects the results of `size` tasks and calls `callback(results)` once, from the thread that
+    delivers the last one (data_transfer.py:18-36)."""
+
+    def __init__(self, size: int, callback: Callable[[list], Any]):
+        self._size = size
+        self._results = [None] * size
+        self._lock = threading.Lock()
+        self._finished_num = 0
+        self._finished_callback = callback
+
+    def submit_result(self, idx: int, result):
+        with self._lock:
+            assert self._results[idx] is None
+            self._results[idx] = result
+            self._finished_num += 1
+            done = self._finished_num == self._size
+        if done:
+            self._finished_callback(self._results)
+
+
+class DataTransferManager:
+    """save_task: wait for the KV cache -> gather blocks into staging slots -> hand the slots to the transfer
+    client. load_task: let the transfer client fill staging slots -> scatter them into the KV cache.
+
+    Stream/event choreography and failure behaviour follow data_transfer.py: one save and one load stream;
+    the gather waits for `kvcache_ready_event`; the calling thread waits for the copy with an event, not a
+    device-wide sync; when the client reports an error on load the scatter is NOT launched (:137-156); staging
+    slots are always returned; every block of a task gets the task's result code.
+    `block_token_indices` may be nested lists (as generate_blocks_idx returns in the reference), a flat list
+    or an int32 tensor.
+    """
+
+    def __init__(self, kvcache_info: KVCacheInfo, manager_block_size: int,
+                 copy_buffer_allocator: CopyBufferAllocator, transfer_client: Any,
+                 client_module: Any = client_types, max_workers: int = 32):
+        self._kvcache_info = kvcache_info
+        self._manager_block_size = manager_block_size
+        self._copy_buffer_allocator = copy_buffer_allocator
+        self._transfer_client = transfer_client
+        self._cm = client_module
+        device = kvcache_info.device
+
+        def init_worker():
+            torch.cuda.set_device(device)
+
+        self._io_executor = ThreadPoolExecutor(max_workers=max_workers, thread_name_prefix="kvcm_io_",
+                                               initializer=init_worker)
+        with torch.cuda.device(device):
+            self._save_stream = torch.cuda.Stream()
+            self._load_stream = torch.cuda.Stream()
+
+    def submit_task(self, func, *args, **kwargs):
+        return self._io_executor.submit(func, *args, **kwargs)
+
+    def shutdown(self):
+        self._io_executor.shutdown(wait=True)
+
+    @staticmethod
+    def _flat_indices(block_token_indices):
+        if isinstance(block_token_indices, torch.Tensor):
+            return block_token_indices
+        if len(block_token_indices) > 0 and isinstance(block_token_indices[0], (list, tuple)):
+            return [t for row in block_token_indices for t in row]
+        return block_token_indices
+
+    def _slot_buffers(self, slot_indices):
+        on_gpu = self._copy_buffer_allocator.device.type != "cpu"
+        mem = self._cm.MemoryType.GPU if on_gpu else self._cm.MemoryType.CPU
+        buffers = []
+        for slot in self._copy_buffer_allocator.get_buffer_by_idx(slot_indices):
+            iov = self._cm.Iov()
+            iov.type = mem
+            iov.base = slot.data_ptr()
+            iov.size = slot.numel() * slot.element_size()
+            iov.ignore = False
+            buf = self._cm.BlockBuffer()
+            buf.iovs = [iov]
+            buffers.append(buf)
+        return buffers
+
+    def load_task(self, multi_result: MultiResult, task_idx: int, remote_uris: List[str], block_token_indices):
+        ok = self._cm.ClientErrorCode.ER_OK
+        slots = self._copy_buffer_allocator.alloc_buffer_idx_blocking(len(remote_uris))
+        try:
+            result = self._transfer_client.LoadKvCaches(remote_uris, self._slot_buffers(slots))
+            if result == ok:
+                with torch.cuda.stream(self._load_stream):
+                    batch_gather_scatter_helper.batch_scatter_kv_caches(
+                        self._kvcache_info.all_kvcache_ptr_tensor_gpu, self._copy_buffer_allocator._raw_buffer,
+                        self._flat_indices(block_token_indices), slots, self._manager_block_size,
+                        self._kvcache_info.per_token_per_layer_dim_size)
+                    done = torch.cuda.Event()
+                    done.record(self._load_stream)
+                done.synchronize()
+        finally:
+            self._copy_buffer_allocator.free_buffer(slots)
+        multi_result.submit_result(task_idx, [result] * len(remote_uris))
+
+    def save_task(self, multi_result: MultiResult, task_idx: int, remote_uris: List[str], block_token_indices,
+                  kvcache_ready_event: Optional[torch.cuda.Event] = None):
+        slots = None
+        try:
+            with torch.cuda.stream(self._save_stream):
+                if kvcache_ready_event is not None:
+                    kvcache_ready_event.wait()
+                slots = self._copy_buffer_allocator.alloc_buffer_idx_blocking(len(remote_uris))
+                batch_gather_scatter_helper.batch_gather_kv_caches(
+                    self._kvcache_info.all_kvcache_ptr_tensor_gpu, self._copy_buffer_allocator._raw_buffer,
+                    self._flat_indices(block_token_indices), slots, self._manager_block_size,
+                    self._kvcache_info.per_token_per_layer_dim_size)
+                done = torch.cuda.Event()
+                done.record(self._save_stream)
+            done.synchronize()
+            result = self._transfer_client.SaveKvCaches(remote_uris, self._slot_buffers(slots))
+        finally:
+            if slots is not None:
+                self._copy_buffer_allocator.free_buffer(slots)
+        multi_result.submit_result(task_idx, [result[0]] * len(remote_uris))

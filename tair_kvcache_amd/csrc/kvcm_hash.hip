@@ -1,0 +1,397 @@
+// kvcm_hash.hip -- block keys of token-ID sequences, batched over requests.
+//
+// Function: GenKeyVector (kv_cache_manager/manager/cache_manager.cc:76-87) over hashInt64Array
+// (kv_cache_manager/manager/hash_util.h:14-24): ONE running 64-bit state per request goes through every
+// token, h <- h ^ (v + C + (h << 12) + (h >> 32)), and is emitted at every block boundary. The step mixes
+// + and ^, so a request is a serial chain of len dependent steps; the parallelism is across requests.
+//
+// Design (gfx950, wave64): a workgroup owns 64 requests and is role-split.
+//   wave 0      "chain wave": lane = request. Keeps the state in VGPRs and does nothing but the
+//               recurrence, reading pre-added terms a = v + C from LDS (one ds_read_b128 per 2 steps).
+//               A single wave issues about one instruction per 4 cycles, so every instruction removed
+//               from this wave shortens the critical path of all 64 chains.
+//   waves 1..3  "loader waves": stream the 64 requests' tokens from HBM in [64 requests x 32 tokens]
+//               tiles with coalesced 256-byte row segments, add C, and write them transposed into a
+//               3-deep LDS ring. Each loader wave owns every third tile and keeps its global loads in
+//               flight for about three tile periods, so HBM latency stays off the chain.
+// Roofline: HBM for many requests (8*block_size + 8 bytes per key); for few requests the bound is the
+// dependent-instruction latency of the chain, which no amount of bandwidth removes.
+#include "kvcm_internal.h"
+
+namespace kvcm {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kReqs = 64;    // requests per workgroup = lanes of the chain wave
+constexpr int kTT = 32;      // tokens per request per tile
+constexpr int kRing = 3;     // LDS tiles in the ring
+constexpr int kPad = 2;      // keeps rows 16-byte aligned (b128 reads) and spreads banks
+constexpr int kLoaders = 3;  // loader waves
+constexpr int kPerLane = kReqs * kTT / 64;  // tile elements per loader lane
+
+// Workgroup barrier that waits only for this wave's LDS traffic. __syncthreads() would also drain the
+// loader waves' outstanding global loads, which must stay in flight across barriers.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <typename TokT>
+__device__ __forceinline__ void issue_tile_loads(uint64_t (&regs)[kPerLane], const TokT *tokens, const int64_t *s_start,
+                                                 const int64_t *s_ntok, int64_t t0, uint32_t lane) {
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j) {
+        const uint32_t e = lane + 64u * j;
+        const uint32_t req = e / kTT;
+        const int64_t g = t0 + (e % kTT);
+        uint64_t a = 0;
+        if (g < s_ntok[req]) {
+            a = static_cast<uint64_t>(static_cast<int64_t>(tokens[s_start[req] + g])) + kGolden;
+        }
+        regs[j] = a;
+    }
+}
+
+__device__ __forceinline__ void store_tile(uint64_t (*tile)[kTT + kPad], const uint64_t (&regs)[kPerLane],
+                                           uint32_t lane) {
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j) {
+        const uint32_t e = lane + 64u * j;
+        tile[e / kTT][e % kTT] = regs[j];
+    }
+}
+
+// CHUNK = steps between two looks at the block boundary: 8 when block_size % 8 == 0 (a lane is then
+// active for whole chunks or not at all), otherwise 1.
+template <typename TokT, int CHUNK>
+__global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__restrict__ tokens,
+                                                              const int64_t *__restrict__ token_offsets, int32_t R,
+                                                              int32_t block_size, uint64_t seed,
+                                                              int64_t *__restrict__ keys,
+                                                              const int64_t *__restrict__ key_offsets) {
+    __shared__ __attribute__((aligned(16))) uint64_t s_tile[kRing][kReqs][kTT + kPad];
+    __shared__ int64_t s_start[kReqs];
+    __shared__ int64_t s_ntok[kReqs];
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * kReqs + lane;
+
+    int64_t my_ntok = 0;
+    if (wave == 0) {
+        int64_t start = 0;
+        if (r < R) {
+            start = token_offsets[r];
+            const int64_t n = token_offsets[r + 1] - start;
+            my_ntok = (n / block_size) * block_size;  // a trailing partial block yields no key
+        }
+        s_start[lane] = start;
+        s_ntok[lane] = my_ntok;
+    }
+    __syncthreads();
+
+    int64_t max_ntok = s_ntok[lane];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const int64_t other = __shfl_xor(max_ntok, o);
+        max_ntok = other > max_ntok ? other : max_ntok;
+    }
+    const int64_t ntiles = (max_ntok + kTT - 1) / kTT;  // uniform over the workgroup
+    if (ntiles == 0) {
+        return;
+    }
+
+    if (wave != 0) {
+        // ---------------------------------------------------------------- loader waves
+        const int64_t lw = wave - 1;
+        uint64_t regs[kPerLane];
+        if (lw < ntiles) {
+            issue_tile_loads(regs, tokens, s_start, s_ntok, lw * kTT, lane);
+        }
+        if (lw == 0) {
+            store_tile(s_tile[0], regs, lane);
+            if (kLoaders < ntiles) {
+                issue_tile_loads(regs, tokens, s_start, s_ntok, static_cast<int64_t>(kLoaders) * kTT, lane);
+            }
+        }
+        lds_barrier();
+        for (int64_t k = 0; k < ntiles; ++k) {
+            const int64_t nxt = k + 1;  // tile that must be in LDS when this iteration ends
+            if (nxt < ntiles && nxt % kLoaders == lw) {
+                store_tile(s_tile[nxt % kRing], regs, lane);
+                if (nxt + kLoaders < ntiles) {
+                    issue_tile_loads(regs, tokens, s_start, s_ntok, (nxt + kLoaders) * kTT, lane);
+                }
+            }
+            lds_barrier();
+        }
+        return;
+    }
+
+    // -------------------------------------------------------------------- chain wave
+    uint64_t h = seed;
+    int64_t key_pos = 0;
+    if (r < R) {
+        key_pos = key_offsets ? key_offsets[r] : r * ((token_offsets[1] - token_offsets[0]) / block_size);
+    }
+    int32_t since_key = 0;  // uniform: all lanes step in lockstep from token 0
+    lds_barrier();
+    for (int64_t k = 0; k < ntiles; ++k) {
+        const uint64_t *row = &s_tile[k % kRing][lane][0];
+        const int64_t t0 = k * kTT;
+#pragma unroll
+        for (int c = 0; c < kTT; c += CHUNK) {
+            const bool active = (t0 + c) < my_ntok;
+            if (active) {
+#pragma unroll
+                for (int s = 0; s < CHUNK; ++s) {
+                    h = hash_step_preadded(h, row[c + s]);
+                }
+            }
+            since_key += CHUNK;
+            if (since_key == block_size) {
+                since_key = 0;
+                if (active) {
+                    keys[key_pos] = static_cast<int64_t>(h);
+                }
+                key_pos += 1;
+            }
+        }
+        lds_barrier();
+    }
+}
+
+// ------------------------------------------------------------------------------------------- SHA-256
+
+__constant__ uint32_t kShaK[64] = {
+    0x428a2f98, 0x71374491, 0xb5c0fbcf, 0xe9b5dba5, 0x3956c25b, 0x59f111f1, 0x923f82a4, 0xab1c5ed5,
+    0xd807aa98, 0x12835b01, 0x243185be, 0x550c7dc3, 0x72be5d74, 0x80deb1fe, 0x9bdc06a7, 0xc19bf174,
+    0xe49b69c1, 0xefbe4786, 0x0fc19dc6, 0x240ca1cc, 0x2de92c6f, 0x4a7484aa, 0x5cb0a9dc, 0x76f988da,
+    0x983e5152, 0xa831c66d, 0xb00327c8, 0xbf597fc7, 0xc6e00bf3, 0xd5a79147, 0x06ca6351, 0x14292967,
+    0x27b70a85, 0x2e1b2138, 0x4d2c6dfc, 0x53380d13, 0x650a7354, 0x766a0abb, 0x81c2c92e, 0x92722c85,
+    0xa2bfe8a1, 0xa81a664b, 0xc24b8b70, 0xc76c51a3, 0xd192e819, 0xd6990624, 0xf40e3585, 0x106aa070,
+    0x19a4c116, 0x1e376c08, 0x2748774c, 0x34b0bcb5, 0x391c0cb3, 0x4ed8aa4a, 0x5b9cca4f, 0x682e6ff3,
+    0x748f82ee, 0x78a5636f, 0x84c87814, 0x8cc70208, 0x90befffa, 0xa4506ceb, 0xbef9a3f7, 0xc67178f2};
+
+__device__ __forceinline__ uint32_t rotr(uint32_t x, int n) { return __builtin_amdgcn_alignbit(x, x, n); }
+
+// One FIPS 180-4 compression; w holds the 16 big-endian message words and is used as the rolling schedule.
+__device__ void sha256_compress(uint32_t (&st)[8], uint32_t (&w)[16]) {
+    uint32_t a = st[0], b = st[1], c = st[2], d = st[3], e = st[4], f = st[5], g = st[6], h = st[7];
+#pragma unroll
+    for (int i = 0; i < 64; ++i) {
+        if (i >= 16) {
+            const uint32_t w15 = w[(i + 1) & 15], w2 = w[(i + 14) & 15];
+            const uint32_t s0 = rotr(w15, 7) ^ rotr(w15, 18) ^ (w15 >> 3);
+            const uint32_t s1 = rotr(w2, 17) ^ rotr(w2, 19) ^ (w2 >> 10);
+            w[i & 15] = w[i & 15] + s0 + w[(i + 9) & 15] + s1;
+        }
+        const uint32_t S1 = rotr(e, 6) ^ rotr(e, 11) ^ rotr(e, 25);
+        const uint32_t ch = (e & f) ^ (~e & g);
+        const uint32_t t1 = h + S1 + ch + kShaK[i] + w[i & 15];
+        const uint32_t S0 = rotr(a, 2) ^ rotr(a, 13) ^ rotr(a, 22);
+        const uint32_t mj = (a & b) ^ (a & c) ^ (b & c);
+        const uint32_t t2 = S0 + mj;
+        h = g;
+        g = f;
+        f = e;
+        e = d + t1;
+        d = c;
+        c = b;
+        b = a;
+        a = t1 + t2;
+    }
+    st[0] += a;
+    st[1] += b;
+    st[2] += c;
+    st[3] += d;
+    st[4] += e;
+    st[5] += f;
+    st[6] += g;
+    st[7] += h;
+}
+
+// Byte i of the padded message of length len: data, 0x80, zeros, 64-bit big-endian bit length.
+__device__ __forceinline__ uint32_t padded_byte(const uint8_t *msg, int64_t len, int64_t padded_len, int64_t i) {
+    if (i < len) {
+        return msg[i];
+    }
+    if (i == len) {
+        return 0x80u;
+    }
+    if (i >= padded_len - 8) {
+        const uint64_t bits = static_cast<uint64_t>(len) * 8u;
+        return static_cast<uint32_t>((bits >> (8 * (padded_len - 1 - i))) & 0xffu);
+    }
+    return 0u;
+}
+
+// One lane per string: key = big-endian signed int64 of SHA-256(bytes)[0:8]
+// (kv_cache_manager/py_connector/sglang/connector.py:397-401).
+__global__ __launch_bounds__(64) void sha256_first8_kernel(const uint8_t *__restrict__ bytes,
+                                                           const int64_t *__restrict__ offsets, int32_t N,
+                                                           int64_t *__restrict__ out) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= N) {
+        return;
+    }
+    const uint8_t *msg = bytes + offsets[i];
+    const int64_t len = offsets[i + 1] - offsets[i];
+    const int64_t padded_len = ((len + 8) / 64 + 1) * 64;
+    uint32_t st[8] = {0x6a09e667, 0xbb67ae85, 0x3c6ef372, 0xa54ff53a, 0x510e527f, 0x9b05688c, 0x1f83d9ab, 0x5be0cd19};
+    for (int64_t base = 0; base < padded_len; base += 64) {
+        uint32_t w[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int64_t p = base + 4 * j;
+            w[j] = (padded_byte(msg, len, padded_len, p) << 24) | (padded_byte(msg, len, padded_len, p + 1) << 16) |
+                   (padded_byte(msg, len, padded_len, p + 2) << 8) | padded_byte(msg, len, padded_len, p + 3);
+        }
+        sha256_compress(st, w);
+    }
+    out[i] = static_cast<int64_t>((static_cast<uint64_t>(st[0]) << 32) | st[1]);
+}
+
+// ------------------------------------------------------------------------------------------- iov CRC-32
+
+// kv_cache_manager/client/src/internal/sdk/sdk_buffer_check_util.cu:10-19.
+__device__ __forceinline__ uint32_t crc32_byte(uint32_t crc, uint8_t data) {
+    crc ^= data;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t mask = 0u - (crc & 1u);
+        crc = (crc >> 1) ^ (0xEDB88320u & mask);
+    }
+    return crc;
+}
+
+// One lane per iov, head bytes then tail bytes through one running CRC (sdk_buffer_check_util.cu:21-44).
+__global__ __launch_bounds__(256) void iov_crc32_kernel(const kvcm_iov_device *__restrict__ iovs, int32_t n,
+                                                        uint32_t *__restrict__ out, size_t cal_bytes) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) {
+        return;
+    }
+    const uint8_t *p = static_cast<const uint8_t *>(iovs[i].base);
+    const size_t size = iovs[i].size;
+    uint32_t crc = 0xFFFFFFFFu;
+    for (size_t k = 0; k < cal_bytes; ++k) {
+        crc = crc32_byte(crc, p[k]);
+    }
+    for (size_t k = size - cal_bytes; k < size; ++k) {
+        crc = crc32_byte(crc, p[k]);
+    }
+    out[i] = ~crc;
+}
+
+template <typename TokT>
+int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_t R, int32_t block_size, int64_t seed,
+                    int64_t *d_keys, const int64_t *d_key_offsets, hipStream_t stream) {
+    if (R < 0 || block_size <= 0) {
+        return KVCM_ERR_INVALID_ARG;
+    }
+    if (R == 0) {
+        return KVCM_OK;
+    }
+    if (!d_tokens || !d_token_offsets || !d_keys) {
+        return KVCM_ERR_INVALID_ARG;
+    }
+    const dim3 grid(static_cast<uint32_t>((static_cast<int64_t>(R) + kReqs - 1) / kReqs));
+    if (block_size % 8 == 0) {
+        hipLaunchKernelGGL((hash_tokens_kernel<TokT, 8>), grid, dim3(kThreads), 0, stream, d_tokens, d_token_offsets, R,
+                           block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets);
+    } else {
+        hipLaunchKernelGGL((hash_tokens_kernel<TokT, 1>), grid, dim3(kThreads), 0, stream, d_tokens, d_token_offsets, R,
+                           block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets);
+    }
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace kvcm
+
+extern "C" {
+
+int32_t kvcm_hip_version(void) { return 100; }
+
+const char *kvcm_hip_error_string(int32_t code) {
+    switch (code) {
+        case KVCM_OK:
+            return "ok";
+        case KVCM_ERR_INVALID_ARG:
+            return "invalid argument";
+        case KVCM_ERR_ALIGNMENT:
+            return "misaligned address or stride";
+        case KVCM_ERR_TOO_LARGE:
+            return "size exceeds the launch geometry";
+        default:
+            return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown kvcm error";
+    }
+}
+
+int32_t kvcm_hip_hash_tokens(const int64_t *d_tokens, const int64_t *d_token_offsets, int32_t R, int32_t block_size,
+                             int64_t seed, int64_t *d_keys, const int64_t *d_key_offsets, kvcm_stream_t stream) {
+    return kvcm::launch_hash<int64_t>(d_tokens, d_token_offsets, R, block_size, seed, d_keys, d_key_offsets,
+                                      static_cast<hipStream_t>(stream));
+}
+
+int32_t kvcm_hip_hash_tokens_i32(const int32_t *d_tokens, const int64_t *d_token_offsets, int32_t R,
+                                 int32_t block_size, int64_t seed, int64_t *d_keys, const int64_t *d_key_offsets,
+                                 kvcm_stream_t stream) {
+    return kvcm::launch_hash<int32_t>(d_tokens, d_token_offsets, R, block_size, seed, d_keys, d_key_offsets,
+                                      static_cast<hipStream_t>(stream));
+}
+
+int32_t kvcm_hip_prefix_chain(const int64_t *d_digests, const int64_t *d_offsets, int32_t R, int64_t *d_keys,
+                              kvcm_stream_t stream) {
+    // ApplyPrefixHash (trace_util.cc:47-56) is the token fold with one element per key: block_size 1,
+    // seed 0, keys laid out like the digests.
+    return kvcm::launch_hash<int64_t>(d_digests, d_offsets, R, 1, 0, d_keys, d_offsets,
+                                      static_cast<hipStream_t>(stream));
+}
+
+int32_t kvcm_hip_sha256_first8_be(const uint8_t *d_bytes, const int64_t *d_offsets, int32_t N, int64_t *d_out,
+                                  kvcm_stream_t stream) {
+    if (N < 0) {
+        return KVCM_ERR_INVALID_ARG;
+    }
+    if (N == 0) {
+        return KVCM_OK;
+    }
+    if (!d_bytes || !d_offsets || !d_out) {
+        return KVCM_ERR_INVALID_ARG;
+    }
+    hipLaunchKernelGGL(kvcm::sha256_first8_kernel, dim3((N + 63) / 64), dim3(64), 0, static_cast<hipStream_t>(stream),
+                       d_bytes, d_offsets, N, d_out);
+    return kvcm::launch_status();
+}
+
+int32_t kvcm_hip_iov_crc32(const kvcm_iov_device *d_iovs, int32_t n, uint32_t *d_crc, size_t cal_bytes,
+                           kvcm_stream_t stream) {
+    if (n < 0) {
+        return KVCM_ERR_INVALID_ARG;
+    }
+    if (n == 0) {
+        return KVCM_OK;
+    }
+    if (!d_iovs || !d_crc) {
+        return KVCM_ERR_INVALID_ARG;
+    }
+    hipLaunchKernelGGL(kvcm::iov_crc32_kernel, dim3((n + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       d_iovs, n, d_crc, cal_bytes);
+    return kvcm::launch_status();
+}
+
+int32_t kvcm_blocks_hash_from_crcs(const uint32_t *crcs, int64_t n_crcs, int32_t iovs_per_block, int64_t *out_hashes) {
+    if (iovs_per_block <= 0 || n_crcs < 0 || (n_crcs > 0 && (!crcs || !out_hashes))) {
+        return KVCM_ERR_INVALID_ARG;
+    }
+    int64_t nb = 0;
+    for (int64_t off = 0; off + iovs_per_block <= n_crcs; off += iovs_per_block) {
+        uint64_t h = 0;
+        for (int32_t i = 0; i < iovs_per_block; ++i) {
+            h = kvcm::hash_step_preadded(h, static_cast<uint64_t>(crcs[off + i]) + kvcm::kGolden);
+        }
+        out_hashes[nb++] = static_cast<int64_t>(h);
+    }
+    return KVCM_OK;
+}
+
+}  // extern "C"

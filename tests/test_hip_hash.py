@@ -1,0 +1,105 @@
+"""GPU parity: block keys from the HIP kernels, through the C-ABI, against the golden vectors and the CPU oracle.
+Bit-exact int64."""
+import hashlib
+
+import numpy as np
+import pytest
+import torch
+
+import _cases as cases
+from _gpu import dev, host, sync
+
+pytestmark = pytest.mark.gpu
+
+
+def _h():
+    from tair_kvcache_amd import hashing
+    return hashing
+
+
+def test_golden_c1(golden):
+    tok = cases.tokens(4, 512, 151936, shared_rows=4, shared_len=256, seed=0)
+    assert tok[0, :8].tolist() == golden["c1"]["tokens_row0_first8"]
+    keys, off = _h().hash_tokens(dev(tok), 16)
+    sync()
+    assert host(off, np.int64).tolist() == [0, 32, 64, 96, 128]
+    assert host(keys, np.int64).reshape(4, 32).tolist() == golden["c1"]["keys"]
+    keys32, _ = _h().hash_tokens(dev(tok.astype(np.int32)), 16)
+    sync()
+    assert host(keys32, np.int64).reshape(4, 32).tolist() == golden["c1"]["keys"]
+
+
+def test_golden_cases_single_requests(golden):
+    for case in golden["cases"]:
+        got = _h().gen_key_vector(case["tokens"], case["block_size"])
+        assert got == case["keys"], case["name"]
+
+
+def test_golden_prefix_chains(golden):
+    for ch in golden["prefix_chains"]:
+        if not ch["ids"]:
+            continue
+        got = _h().apply_prefix_hash(torch.tensor(ch["ids"], dtype=torch.int64, device="cuda"))
+        sync()
+        assert got.tolist() == ch["keys"]
+
+
+@pytest.mark.parametrize("R,L,bs", [(64, 4096, 16), (1, 16, 16), (3, 1000, 16), (65, 256, 64), (130, 96, 8),
+                                    (32, 1024, 128), (7, 333, 7), (5, 64, 1), (200, 40, 24)])
+def test_uniform_batches_match_oracle(oracle, R, L, bs):
+    print(f"hash case R={R} L={L} bs={bs}", flush=True)
+    rng = np.random.default_rng(R * 1000 + L + bs)
+    tok = rng.integers(-2**63, 2**63 - 1, size=(R, L), dtype=np.int64)  # full int64 range, both signs
+    want, woff = oracle.hash_tokens(tok, bs)
+    keys, off = _h().hash_tokens(dev(tok), bs)
+    sync()
+    assert (host(off, np.int64) == woff).all()
+    assert (host(keys, np.int64) == want).all()
+
+
+def test_ragged_batch_and_seed(oracle):
+    rng = np.random.default_rng(3)
+    lens = [0, 5, 16, 17, 160, 33, 1024, 31, 4096, 15, 48] + [int(x) for x in rng.integers(0, 700, size=120)]
+    toks = [rng.integers(0, 152064, size=n, dtype=np.int64) for n in lens]
+    flat = np.concatenate(toks)
+    toff = np.zeros(len(lens) + 1, dtype=np.int64)
+    np.cumsum(lens, out=toff[1:])
+    for bs, seed in [(16, 0), (16, 12345), (5, -7), (64, 0)]:
+        want, woff = oracle.hash_tokens(flat, bs, token_offsets=toff, seed=seed)
+        keys, off = _h().hash_tokens(dev(flat), bs, token_offsets=dev(toff), seed=seed)
+        sync()
+        assert (host(off, np.int64) == woff).all()
+        assert (host(keys, np.int64) == want).all(), (bs, seed)
+
+
+def test_config2_batch_prefix_property(oracle):
+    """64 x 4096 tokens, half the requests share a 2048-token prefix: 128 leading keys shared, the rest distinct."""
+    tok = cases.tokens(64, 4096, 128256, shared_rows=32, shared_len=2048, seed=0)
+    keys, _ = _h().hash_tokens(dev(tok), 16)
+    sync()
+    k = host(keys, np.int64).reshape(64, 256)
+    want, _ = oracle.hash_tokens(tok, 16)
+    assert (k == want.reshape(64, 256)).all()
+    assert (k[:32, :128] == k[0, :128]).all()
+    assert len(np.unique(k[:, 128])) == 64 and len(np.unique(k[32:, 0])) == 32
+
+
+def test_config5_many_requests(oracle):
+    tok = cases.tokens(1024, 1024, 152064, seed=0)
+    keys, _ = _h().hash_tokens(dev(tok), 16)
+    sync()
+    want, _ = oracle.hash_tokens(tok, 16, threads=8)
+    assert (host(keys, np.int64) == want).all()
+
+
+def test_sha256_keys(oracle):
+    rng = np.random.default_rng(6)
+    strs = ["", "abc", "é-ü-漢字", "x" * 55, "y" * 56, "z" * 64, "w" * 119, "v" * 120, "u" * 1000]
+    strs += ["%064x" % int(x) for x in rng.integers(0, 2**62, size=300)]
+    got = _h().sha256_to_int64(strs).tolist()
+    want = [int.from_bytes(hashlib.sha256(s.encode("utf-8")).digest()[:8], "big", signed=True) for s in strs]
+    assert got == want
+    assert got == oracle.sha256_first8_be(strs).tolist()
+    keys, n_prefix, n_new = _h().prepare_block_keys(strs[10:20], prefix_keys=strs[:3])
+    assert (n_prefix, n_new) == (3, 10) and keys == want[:3] + want[10:20]
+    assert _h().prepare_block_keys([], None) == ([], 0, 0)

@@ -1,0 +1,144 @@
+"""GPU parity: buffer check (iov CRC + block fold) and the save/load choreography around the kernels."""
+import threading
+import zlib
+
+import numpy as np
+import pytest
+import torch
+
+import _cases as cases
+from _gpu import dev, host, ptr_table, sync
+
+pytestmark = pytest.mark.gpu
+
+
+def test_iov_crc_reference_known_answers():
+    # kv_cache_manager/client/src/internal/sdk/test/sdk_buffer_check_util_test.cc:13-74
+    from tair_kvcache_amd import buffer_check as bc
+    s = torch.frombuffer(bytearray(b"1234xxxxxxxx5678"), dtype=torch.uint8).cuda()
+    assert bc.get_iovs_crc([(s.data_ptr(), 16)], cal_byte_size=8) == [0xDE28307C]
+    assert bc.get_iovs_crc([(s.data_ptr(), 16)], cal_byte_size=4) == [0x9AE0DAAF]
+    s2 = torch.frombuffer(bytearray(b"1278"), dtype=torch.uint8).cuda()
+    assert bc.get_iovs_crc([(s2.data_ptr(), 4)], cal_byte_size=4) == [0xF639698C]
+    s3 = torch.frombuffer(bytearray(b"1"), dtype=torch.uint8).cuda()
+    assert bc.get_iovs_crc([(s3.data_ptr(), 1)], cal_byte_size=4) == []
+
+
+def test_iov_crc_and_block_hash_match_oracle(oracle):
+    from tair_kvcache_amd import buffer_check as bc
+    rng = np.random.default_rng(8)
+    data = rng.integers(0, 256, size=(6, 4, 1024), dtype=np.uint8)  # 6 blocks x 4 iovs
+    d = dev(data)
+    blocks = [[(d[b, i].data_ptr(), 1024) for i in range(4)] for b in range(6)]
+    flat = [iov for bb in blocks for iov in bb]
+    crcs = bc.get_iovs_crc(flat)
+    want = [zlib.crc32(data[b, i, :4].tobytes() + data[b, i, -4:].tobytes()) for b in range(6) for i in range(4)]
+    assert crcs == want
+    assert crcs == oracle.iov_crc32([data[b, i] for b in range(6) for i in range(4)], 4).tolist()
+    hashes = bc.get_blocks_hash(blocks)
+    assert hashes == oracle.blocks_hash_from_crcs(np.array(want, dtype=np.uint32), 4).tolist()
+    assert len(bc.get_blocks_hash(blocks, max_iov_num=10)) == 2  # whole blocks only (.cc:43-47)
+    same = bc.get_blocks_hash([blocks[0], blocks[0]])
+    assert same[0] == same[1]
+
+
+class FakeTransferClient:
+    """Keeps blocks in a dict keyed by URI; stands in for TransferClient (transfer_client.h:19-21)."""
+
+    def __init__(self, fail_load=False):
+        self.store = {}
+        self.fail_load = fail_load
+        self.lock = threading.Lock()
+
+    def SaveKvCaches(self, uris, buffers):
+        from tair_kvcache_amd.client_types import ClientErrorCode
+        if len(uris) != len(buffers) or not uris:
+            return (ClientErrorCode.ER_INVALID_PARAMS, [])
+        import ctypes
+        with self.lock:
+            for uri, buf in zip(uris, buffers):
+                iov = buf.iovs[0]
+                self.store[uri] = ctypes.string_at(iov.base, iov.size)
+        return (ClientErrorCode.ER_OK, list(uris))
+
+    def LoadKvCaches(self, uris, buffers):
+        from tair_kvcache_amd.client_types import ClientErrorCode
+        if self.fail_load:
+            return ClientErrorCode.ER_SDKREAD_ERROR
+        import ctypes
+        for uri, buf in zip(uris, buffers):
+            iov = buf.iovs[0]
+            ctypes.memmove(iov.base, self.store[uri], iov.size)
+        return ClientErrorCode.ER_OK
+
+
+def test_save_then_load_through_the_transfer_manager(oracle):
+    """register_kv_caches -> generate_blocks_idx -> save_task (gather + client) -> load_task (client + scatter) on
+    vLLM-shaped caches [2, blocks, block_size, heads, dim]; stored bytes equal the oracle's staging layout."""
+    from tair_kvcache_amd import connector
+    from tair_kvcache_amd.client_types import ClientErrorCode
+    from tair_kvcache_amd.kernel.gather_scatter_helper import CopyBufferAllocator
+    L, nblk, T, H, hd = 4, 64, 16, 2, 64
+    rng = np.random.default_rng(1)
+    np_caches = [rng.integers(0, 65536, size=(2, nblk, T, H, hd), dtype=np.uint16) for _ in range(L)]
+    kv = {f"layer{l}": dev(np_caches[l]).view(torch.bfloat16) for l in range(L)}
+    info = connector.register_kv_caches(kv, manager_block_size=T, local_block_size=T)
+    assert info.per_manager_location_spec_shape == (L, 2, T, H * hd)
+    assert info.per_manager_location_spec_byte_size == L * 2 * T * H * hd * 2
+    assert info.all_kvcache_ptr_tensor_gpu.tolist() == [x for l in range(L) for x in
+                                                        (kv[f"layer{l}"][0].data_ptr(), kv[f"layer{l}"][1].data_ptr())]
+    alloc = CopyBufferAllocator(torch.device("cpu"), torch.bfloat16, list(info.per_manager_location_spec_shape), 32)
+    client = FakeTransferClient()
+    mgr = connector.DataTransferManager(info, T, alloc, client, max_workers=4)
+    local_block_ids = cases.block_table(nblk, 24).tolist()
+    manager_blocks = list(range(24))
+    idx = connector.generate_blocks_idx(manager_blocks, local_block_ids, T, T)
+    sync()
+    idx_h = host(idx, np.int32)
+    done = threading.Event()
+    results = []
+    multi = connector.MultiResult(2, lambda r: (results.append(r), done.set()))
+    ready = torch.cuda.Event()
+    ready.record()
+    uris = [f"file:///kv/blk?blkid={i}&size={info.per_manager_location_spec_byte_size}" for i in range(24)]
+    mgr.submit_task(mgr.save_task, multi, 0, uris[:12], idx_h[:12].tolist(), ready)
+    mgr.submit_task(mgr.save_task, multi, 1, uris[12:], idx[12:], ready)
+    assert done.wait(60)
+    assert results[0] == [[ClientErrorCode.ER_OK] * 12] * 2
+    assert alloc._inuse_count == 0
+    # stored bytes = oracle staging
+    pools = [np_caches[l][kvi].reshape(nblk * T, H * hd) for l in range(L) for kvi in (0, 1)]
+    want = np.zeros((24, 2 * L, T, H * hd), dtype=np.uint16)
+    oracle.batch_gather(pools, want, idx_h, None, T, H * hd * 2)
+    for i, uri in enumerate(uris):
+        assert client.store[uri] == want[i].tobytes()
+    # load into zeroed caches
+    kv2 = {k: torch.zeros_like(v) for k, v in kv.items()}
+    info2 = connector.register_kv_caches(kv2, T, T)
+    mgr2 = connector.DataTransferManager(info2, T, alloc, client, max_workers=4)
+    done2 = threading.Event()
+    res2 = []
+    multi2 = connector.MultiResult(1, lambda r: (res2.append(r), done2.set()))
+    mgr2.submit_task(mgr2.load_task, multi2, 0, uris, idx_h.tolist())
+    assert done2.wait(60)
+    assert res2[0] == [[ClientErrorCode.ER_OK] * 24]
+    touched = np.array(local_block_ids)
+    rest = np.setdiff1d(np.arange(nblk), touched)
+    for l in range(L):
+        g = host(kv2[f"layer{l}"].view(torch.int16), np.uint16)
+        assert (g[:, touched] == np_caches[l][:, touched]).all()
+        assert not g[:, rest].any()
+    # a failed load launches no scatter and still returns the slots
+    kv3 = {k: torch.zeros_like(v) for k, v in kv.items()}
+    mgr3 = connector.DataTransferManager(connector.register_kv_caches(kv3, T, T), T, alloc,
+                                         FakeTransferClient(fail_load=True), max_workers=2)
+    done3 = threading.Event()
+    res3 = []
+    mgr3.submit_task(mgr3.load_task, connector.MultiResult(1, lambda r: (res3.append(r), done3.set())), 0, uris[:4],
+                     idx_h[:4].tolist())
+    assert done3.wait(60)
+    assert res3[0] == [[ClientErrorCode.ER_SDKREAD_ERROR] * 4] and alloc._inuse_count == 0
+    sync()
+    assert all(not v.view(torch.int16).any() for v in kv3.values())
+    for m in (mgr, mgr2, mgr3):
+        m.shutdown()
