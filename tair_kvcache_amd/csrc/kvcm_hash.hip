@@ -33,28 +33,28 @@ constexpr int kPerLane = kReqs * kTT / 64;  // tile elements per loader lane
 // loader waves' outstanding global loads, which must stay in flight across barriers.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// Issues the global loads of one tile without waiting for them. Every address is valid: positions
+// beyond a request's last hashed token are clamped to the last token of the whole batch, and the chain
+// wave never consumes those entries.
 template <typename TokT>
-__device__ __forceinline__ void issue_tile_loads(uint64_t (&regs)[kPerLane], const TokT *tokens, const int64_t *s_start,
-                                                 const int64_t *s_ntok, int64_t t0, uint32_t lane) {
+__device__ __forceinline__ void issue_tile_loads(TokT (&regs)[kPerLane], const TokT *tokens, const int64_t *s_start,
+                                                 int64_t last_token, int64_t t0, uint32_t lane) {
 #pragma unroll
     for (int j = 0; j < kPerLane; ++j) {
         const uint32_t e = lane + 64u * j;
-        const uint32_t req = e / kTT;
-        const int64_t g = t0 + (e % kTT);
-        uint64_t a = 0;
-        if (g < s_ntok[req]) {
-            a = static_cast<uint64_t>(static_cast<int64_t>(tokens[s_start[req] + g])) + kGolden;
-        }
-        regs[j] = a;
+        const int64_t pos = s_start[e / kTT] + t0 + (e % kTT);
+        regs[j] = tokens[pos < last_token ? pos : last_token];
     }
 }
 
-__device__ __forceinline__ void store_tile(uint64_t (*tile)[kTT + kPad], const uint64_t (&regs)[kPerLane],
+// Adds the golden-ratio constant (the token term of the step is v + C) and writes the tile transposed.
+template <typename TokT>
+__device__ __forceinline__ void store_tile(uint64_t (*tile)[kTT + kPad], const TokT (&regs)[kPerLane],
                                            uint32_t lane) {
 #pragma unroll
     for (int j = 0; j < kPerLane; ++j) {
         const uint32_t e = lane + 64u * j;
-        tile[e / kTT][e % kTT] = regs[j];
+        tile[e / kTT][e % kTT] = static_cast<uint64_t>(static_cast<int64_t>(regs[j])) + kGolden;
     }
 }
 
@@ -97,35 +97,45 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     if (ntiles == 0) {
         return;
     }
+    const int64_t last_token = token_offsets[R] - 1;  // >= 0 here: some request has a full block
 
     if (wave != 0) {
         // ---------------------------------------------------------------- loader waves
         const int64_t lw = wave - 1;
-        uint64_t regs[kPerLane];
+        TokT regs[kPerLane];
         if (lw < ntiles) {
-            issue_tile_loads(regs, tokens, s_start, s_ntok, lw * kTT, lane);
+            issue_tile_loads(regs, tokens, s_start, last_token, lw * kTT, lane);
         }
         if (lw == 0) {
             store_tile(s_tile[0], regs, lane);
-            if (kLoaders < ntiles) {
-                issue_tile_loads(regs, tokens, s_start, s_ntok, static_cast<int64_t>(kLoaders) * kTT, lane);
-            }
         }
         lds_barrier();
+        // Issuing a tile's loads costs a few hundred instruction slots; it happens AFTER the barrier, while the
+        // chain wave is busy with the tile just published, so it never delays the chain.
+        if (lw == 0 && kLoaders < ntiles) {
+            issue_tile_loads(regs, tokens, s_start, last_token, static_cast<int64_t>(kLoaders) * kTT, lane);
+        }
+        static_assert(kRing == kLoaders, "loader lw always fills ring slot lw");
+        int64_t turn = 1 % kLoaders;  // loader whose tile is due: (k + 1) % kLoaders
         for (int64_t k = 0; k < ntiles; ++k) {
             const int64_t nxt = k + 1;  // tile that must be in LDS when this iteration ends
-            if (nxt < ntiles && nxt % kLoaders == lw) {
-                store_tile(s_tile[nxt % kRing], regs, lane);
-                if (nxt + kLoaders < ntiles) {
-                    issue_tile_loads(regs, tokens, s_start, s_ntok, (nxt + kLoaders) * kTT, lane);
-                }
+            const bool mine = turn == lw && nxt < ntiles;
+            turn = turn + 1 == kLoaders ? 0 : turn + 1;
+            if (mine) {
+                store_tile(s_tile[lw], regs, lane);
             }
             lds_barrier();
+            if (mine && nxt + kLoaders < ntiles) {
+                issue_tile_loads(regs, tokens, s_start, last_token, (nxt + kLoaders) * kTT, lane);
+            }
         }
         return;
     }
 
     // -------------------------------------------------------------------- chain wave
+    // A single wave issues one VALU instruction per ~4.8 cycles whether or not it depends on the previous
+    // one (measured), so the step costs its instruction count: the compiler's 7 (v_lshlrev_b64, v_ashrrev_i32,
+    // v_mov, 2 x v_lshl_add_u64, 2 x v_xor_b32) beat a hand-written 9-instruction 32-bit form.
     uint64_t h = seed;
     int64_t key_pos = 0;
     if (r < R) {
@@ -133,16 +143,24 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     }
     int32_t since_key = 0;  // uniform: all lanes step in lockstep from token 0
     lds_barrier();
+    int ring = 0;
     for (int64_t k = 0; k < ntiles; ++k) {
-        const uint64_t *row = &s_tile[k % kRing][lane][0];
+        // the lane's 32 pre-added terms of this tile: 16 ds_read_b128, issued together
+        const ulonglong2 *row = reinterpret_cast<const ulonglong2 *>(&s_tile[ring][lane][0]);
+        ulonglong2 a[kTT / 2];
+#pragma unroll
+        for (int i = 0; i < kTT / 2; ++i) {
+            a[i] = row[i];
+        }
+        ring = ring + 1 == kRing ? 0 : ring + 1;
         const int64_t t0 = k * kTT;
 #pragma unroll
         for (int c = 0; c < kTT; c += CHUNK) {
             const bool active = (t0 + c) < my_ntok;
             if (active) {
 #pragma unroll
-                for (int s = 0; s < CHUNK; ++s) {
-                    h = hash_step_preadded(h, row[c + s]);
+                for (int s = c; s < c + CHUNK; ++s) {
+                    h = hash_step_preadded(h, (s & 1) ? a[s / 2].y : a[s / 2].x);
                 }
             }
             since_key += CHUNK;
