@@ -18,6 +18,8 @@
 // dependent-instruction latency of the chain, which no amount of bandwidth removes.
 #include "kvcm_internal.h"
 
+#include <cstdlib>
+
 namespace kvcm {
 namespace {
 
@@ -33,28 +35,167 @@ constexpr int kPerLane = kReqs * kTT / 64;  // tile elements per loader lane
 // loader waves' outstanding global loads, which must stay in flight across barriers.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// Issues the global loads of one tile without waiting for them. Every address is valid: positions
-// beyond a request's last hashed token are clamped to the last token of the whole batch, and the chain
-// wave never consumes those entries.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// What a loader wave needs to know about its workgroup.
 template <typename TokT>
-__device__ __forceinline__ void issue_tile_loads(TokT (&regs)[kPerLane], const TokT *tokens, const int64_t *s_start,
-                                                 int64_t last_token, int64_t t0, uint32_t lane) {
+struct LoaderCtx {
+    const TokT *tokens;
+    const int64_t *s_start;  // LDS: first token of each of the 64 requests
+    int64_t last_token;      // index of the last token of the whole batch (clamp target)
+    int64_t wg_first_token;  // first token of the workgroup's first request
+    uint32_t wg_bytes;       // bytes from there to the end of the batch, saturated at 2^32 - 1
+};
+
+// Loader, fast form: 16-byte BUFFER loads. One load instruction covers 64 / kLPR request rows with kLPR lanes
+// each, so a tile takes kNL loads per lane (16 for int64 tokens, 8 for int32). The buffer resource spans from the
+// workgroup's first token to the end of the batch: the hardware returns zeros past the end instead of faulting, so
+// the loads need no clamp, and a load costs two instructions (offset add + buffer_load_dwordx4). Positions past a
+// request's own last hashed token read a neighbour's tokens; the chain wave never consumes those entries.
+template <typename TokT>
+struct BufferLoader {
+    static constexpr int kEPL = 16 / sizeof(TokT);  // tokens per load
+    static constexpr int kLPR = kTT / kEPL;         // lanes per request row
+    static constexpr int kRPW = 64 / kLPR;          // request rows per load instruction
+    static constexpr int kNL = kReqs / kRPW;        // loads per lane per tile
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint32_t rel[kNL];  // byte offset of this lane's piece of row j, tile 0
+    u32x4 regs[kNL];
+    uint32_t lane;
+
+    __device__ __forceinline__ void setup(const LoaderCtx<TokT> &c, uint32_t lane_) {
+        lane = lane_;
+        rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<TokT *>(c.tokens + c.wg_first_token), 0, c.wg_bytes,
+                                                 0x00020000);
+        const uint32_t sub = lane / kLPR, piece = lane % kLPR;
 #pragma unroll
-    for (int j = 0; j < kPerLane; ++j) {
-        const uint32_t e = lane + 64u * j;
-        const int64_t pos = s_start[e / kTT] + t0 + (e % kTT);
-        regs[j] = tokens[pos < last_token ? pos : last_token];
+        for (int j = 0; j < kNL; ++j) {
+            rel[j] = static_cast<uint32_t>((c.s_start[j * kRPW + sub] - c.wg_first_token) * sizeof(TokT)) + piece * 16u;
+        }
+    }
+    __device__ __forceinline__ void issue(int64_t t0) {
+        const uint32_t tile_off = static_cast<uint32_t>(t0 * sizeof(TokT));
+#pragma unroll
+        for (int j = 0; j < kNL; ++j) {
+            regs[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, rel[j] + tile_off, 0, 0);
+        }
+    }
+    // Adds the golden-ratio constant (the token term of the step is v + C) and writes the tile transposed.
+    __device__ __forceinline__ void store(uint64_t (*tile)[kTT + kPad]) const {
+        const uint32_t sub = lane / kLPR, piece = lane % kLPR;
+#pragma unroll
+        for (int j = 0; j < kNL; ++j) {
+            ulonglong2 *dst = reinterpret_cast<ulonglong2 *>(&tile[j * kRPW + sub][piece * kEPL]);
+            const u32x4 v = regs[j];
+            if (sizeof(TokT) == 8) {
+                dst[0] = make_ulonglong2(((static_cast<uint64_t>(v.y) << 32) | v.x) + kGolden,
+                                         ((static_cast<uint64_t>(v.w) << 32) | v.z) + kGolden);
+            } else {
+                dst[0] = make_ulonglong2(static_cast<uint64_t>(static_cast<int64_t>(static_cast<int32_t>(v.x))) + kGolden,
+                                         static_cast<uint64_t>(static_cast<int64_t>(static_cast<int32_t>(v.y))) + kGolden);
+                dst[1] = make_ulonglong2(static_cast<uint64_t>(static_cast<int64_t>(static_cast<int32_t>(v.z))) + kGolden,
+                                         static_cast<uint64_t>(static_cast<int64_t>(static_cast<int32_t>(v.w))) + kGolden);
+            }
+        }
+    }
+};
+
+// Loader, general form: one element per load through global addresses, positions clamped to the last token of
+// the batch. Used when the workgroup's requests span 4 GiB or more, which a 32-bit buffer offset cannot address.
+template <typename TokT>
+struct GlobalLoader {
+    LoaderCtx<TokT> c;
+    TokT regs[kPerLane];
+    uint32_t lane;
+
+    __device__ __forceinline__ void setup(const LoaderCtx<TokT> &c_, uint32_t lane_) {
+        c = c_;
+        lane = lane_;
+    }
+    __device__ __forceinline__ void issue(int64_t t0) {
+#pragma unroll
+        for (int j = 0; j < kPerLane; ++j) {
+            const uint32_t e = lane + 64u * j;
+            const int64_t pos = c.s_start[e / kTT] + t0 + (e % kTT);
+            regs[j] = c.tokens[pos < c.last_token ? pos : c.last_token];
+        }
+    }
+    __device__ __forceinline__ void store(uint64_t (*tile)[kTT + kPad]) const {
+#pragma unroll
+        for (int j = 0; j < kPerLane; ++j) {
+            const uint32_t e = lane + 64u * j;
+            tile[e / kTT][e % kTT] = static_cast<uint64_t>(static_cast<int64_t>(regs[j])) + kGolden;
+        }
+    }
+};
+
+// A loader wave's whole life. Loader lw owns tiles lw, lw + 3, ... and ring slot lw. Tiles 0 and 1 are published
+// before the first barrier: the chain wave computes on tile k while its LDS reads of tile k+1 are already in
+// flight, so tile k+2 is what gets written during iteration k. Loads are issued AFTER a barrier, while the chain
+// wave is busy, and stay in flight for about two tile periods.
+template <typename Loader, typename TokT>
+__device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t (*s_tile)[kReqs][kTT + kPad],
+                                           int64_t lw, int64_t ntiles, uint32_t lane) {
+    static_assert(kRing == kLoaders, "loader lw always fills ring slot lw");
+    Loader ld;
+    ld.setup(ctx, lane);
+    if (lw < ntiles) {
+        ld.issue(lw * kTT);
+    }
+    if (lw < 2 && lw < ntiles) {
+        ld.store(s_tile[lw]);
+    }
+    lds_barrier();
+    if (lw < 2 && lw + kLoaders < ntiles) {
+        ld.issue((lw + kLoaders) * kTT);
+    }
+    int64_t turn = 2 % kLoaders;  // loader whose tile is due: (k + 2) % kLoaders
+    for (int64_t k = 0; k < ntiles; ++k) {
+        const int64_t nxt = k + 2;  // tile that must be in LDS when this iteration ends
+        const bool mine = turn == lw && nxt < ntiles;
+        turn = turn + 1 == kLoaders ? 0 : turn + 1;
+        if (mine) {
+            ld.store(s_tile[lw]);
+        }
+        lds_barrier();
+        if (mine && nxt + kLoaders < ntiles) {
+            ld.issue((nxt + kLoaders) * kTT);
+        }
     }
 }
 
-// Adds the golden-ratio constant (the token term of the step is v + C) and writes the tile transposed.
-template <typename TokT>
-__device__ __forceinline__ void store_tile(uint64_t (*tile)[kTT + kPad], const TokT (&regs)[kPerLane],
-                                           uint32_t lane) {
+// The chain wave's work on one tile: kTT steps from the lane's pre-added terms `a`, a key at every block
+// boundary. MASKED = some lane may have run out of tokens inside this tile (ragged batch); the common case of
+// equally long requests takes the unmasked path, which has no per-lane compare in it.
+template <int CHUNK, bool MASKED>
+__device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_t &h, int64_t t0, int64_t my_ntok,
+                                         int32_t &since_key, int32_t block_size, int64_t *__restrict__ keys,
+                                         int64_t &key_pos) {
 #pragma unroll
-    for (int j = 0; j < kPerLane; ++j) {
-        const uint32_t e = lane + 64u * j;
-        tile[e / kTT][e % kTT] = static_cast<uint64_t>(static_cast<int64_t>(regs[j])) + kGolden;
+    for (int c = 0; c < kTT; c += CHUNK) {
+        const bool active = !MASKED || (t0 + c) < my_ntok;
+        if (active) {
+#pragma unroll
+            for (int s = c; s < c + CHUNK; ++s) {
+                h = hash_step_preadded(h, (s & 1) ? a[s / 2].y : a[s / 2].x);
+            }
+        }
+        since_key += CHUNK;
+        if (since_key == block_size) {
+            since_key = 0;
+            if (active) {
+                keys[key_pos] = static_cast<int64_t>(h);
+            }
+            key_pos += 1;
+        }
+    }
+}
+
+__device__ __forceinline__ void read_row(ulonglong2 (&a)[kTT / 2], const uint64_t *row_ptr) {
+    const ulonglong2 *row = reinterpret_cast<const ulonglong2 *>(row_ptr);
+#pragma unroll
+    for (int i = 0; i < kTT / 2; ++i) {
+        a[i] = row[i];
     }
 }
 
@@ -65,7 +206,8 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
                                                               const int64_t *__restrict__ token_offsets, int32_t R,
                                                               int32_t block_size, uint64_t seed,
                                                               int64_t *__restrict__ keys,
-                                                              const int64_t *__restrict__ key_offsets) {
+                                                              const int64_t *__restrict__ key_offsets,
+                                                              int32_t force_global_loads) {
     __shared__ __attribute__((aligned(16))) uint64_t s_tile[kRing][kReqs][kTT + kPad];
     __shared__ int64_t s_start[kReqs];
     __shared__ int64_t s_ntok[kReqs];
@@ -76,7 +218,7 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
 
     int64_t my_ntok = 0;
     if (wave == 0) {
-        int64_t start = 0;
+        int64_t start = token_offsets[static_cast<int64_t>(blockIdx.x) * kReqs];  // rows past R idle at the first row
         if (r < R) {
             start = token_offsets[r];
             const int64_t n = token_offsets[r + 1] - start;
@@ -88,46 +230,36 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     __syncthreads();
 
     int64_t max_ntok = s_ntok[lane];
+    int64_t min_ntok = max_ntok;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
-        const int64_t other = __shfl_xor(max_ntok, o);
-        max_ntok = other > max_ntok ? other : max_ntok;
+        const int64_t hi_other = __shfl_xor(max_ntok, o);
+        const int64_t lo_other = __shfl_xor(min_ntok, o);
+        max_ntok = hi_other > max_ntok ? hi_other : max_ntok;
+        min_ntok = lo_other < min_ntok ? lo_other : min_ntok;
     }
     const int64_t ntiles = (max_ntok + kTT - 1) / kTT;  // uniform over the workgroup
     if (ntiles == 0) {
         return;
     }
-    const int64_t last_token = token_offsets[R] - 1;  // >= 0 here: some request has a full block
 
     if (wave != 0) {
         // ---------------------------------------------------------------- loader waves
-        const int64_t lw = wave - 1;
-        TokT regs[kPerLane];
-        if (lw < ntiles) {
-            issue_tile_loads(regs, tokens, s_start, last_token, lw * kTT, lane);
-        }
-        if (lw == 0) {
-            store_tile(s_tile[0], regs, lane);
-        }
-        lds_barrier();
-        // Issuing a tile's loads costs a few hundred instruction slots; it happens AFTER the barrier, while the
-        // chain wave is busy with the tile just published, so it never delays the chain.
-        if (lw == 0 && kLoaders < ntiles) {
-            issue_tile_loads(regs, tokens, s_start, last_token, static_cast<int64_t>(kLoaders) * kTT, lane);
-        }
-        static_assert(kRing == kLoaders, "loader lw always fills ring slot lw");
-        int64_t turn = 1 % kLoaders;  // loader whose tile is due: (k + 1) % kLoaders
-        for (int64_t k = 0; k < ntiles; ++k) {
-            const int64_t nxt = k + 1;  // tile that must be in LDS when this iteration ends
-            const bool mine = turn == lw && nxt < ntiles;
-            turn = turn + 1 == kLoaders ? 0 : turn + 1;
-            if (mine) {
-                store_tile(s_tile[lw], regs, lane);
-            }
-            lds_barrier();
-            if (mine && nxt + kLoaders < ntiles) {
-                issue_tile_loads(regs, tokens, s_start, last_token, (nxt + kLoaders) * kTT, lane);
-            }
+        LoaderCtx<TokT> ctx;
+        ctx.tokens = tokens;
+        ctx.s_start = s_start;
+        const int64_t total = token_offsets[R];
+        ctx.last_token = total - 1;  // >= 0 here: some request has a full block
+        const int64_t r_first = static_cast<int64_t>(blockIdx.x) * kReqs;
+        const int64_t r_end = r_first + kReqs < R ? r_first + kReqs : R;
+        ctx.wg_first_token = token_offsets[r_first];
+        const uint64_t to_end = static_cast<uint64_t>(total - ctx.wg_first_token) * sizeof(TokT);
+        ctx.wg_bytes = to_end > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(to_end);
+        const uint64_t wg_span = static_cast<uint64_t>(token_offsets[r_end] - ctx.wg_first_token) * sizeof(TokT);
+        if (!force_global_loads && wg_span < 0xFFF00000ull) {
+            run_loader<BufferLoader<TokT>, TokT>(ctx, s_tile, wave - 1, ntiles, lane);
+        } else {
+            run_loader<GlobalLoader<TokT>, TokT>(ctx, s_tile, wave - 1, ntiles, lane);
         }
         return;
     }
@@ -143,34 +275,32 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     }
     int32_t since_key = 0;  // uniform: all lanes step in lockstep from token 0
     lds_barrier();
+    ulonglong2 cur[kTT / 2], nxt[kTT / 2];
+    read_row(cur, &s_tile[0][lane][0]);
     int ring = 0;
-    for (int64_t k = 0; k < ntiles; ++k) {
-        // the lane's 32 pre-added terms of this tile: 16 ds_read_b128, issued together
-        const ulonglong2 *row = reinterpret_cast<const ulonglong2 *>(&s_tile[ring][lane][0]);
-        ulonglong2 a[kTT / 2];
-#pragma unroll
-        for (int i = 0; i < kTT / 2; ++i) {
-            a[i] = row[i];
+    for (int64_t k = 0; k < ntiles; k += 2) {
+        // even tile: compute on `cur`, prefetch the odd tile into `nxt`; then the other way round
+        int ring1 = ring + 1 == kRing ? 0 : ring + 1;
+        if (k + 1 < ntiles) {
+            read_row(nxt, &s_tile[ring1][lane][0]);
         }
-        ring = ring + 1 == kRing ? 0 : ring + 1;
-        const int64_t t0 = k * kTT;
-#pragma unroll
-        for (int c = 0; c < kTT; c += CHUNK) {
-            const bool active = (t0 + c) < my_ntok;
-            if (active) {
-#pragma unroll
-                for (int s = c; s < c + CHUNK; ++s) {
-                    h = hash_step_preadded(h, (s & 1) ? a[s / 2].y : a[s / 2].x);
-                }
-            }
-            since_key += CHUNK;
-            if (since_key == block_size) {
-                since_key = 0;
-                if (active) {
-                    keys[key_pos] = static_cast<int64_t>(h);
-                }
-                key_pos += 1;
-            }
+        if ((k + 1) * kTT <= min_ntok) {
+            run_tile<CHUNK, false>(cur, h, k * kTT, my_ntok, since_key, block_size, keys, key_pos);
+        } else {
+            run_tile<CHUNK, true>(cur, h, k * kTT, my_ntok, since_key, block_size, keys, key_pos);
+        }
+        lds_barrier();
+        if (k + 1 >= ntiles) {
+            break;
+        }
+        ring = ring1 + 1 == kRing ? 0 : ring1 + 1;
+        if (k + 2 < ntiles) {
+            read_row(cur, &s_tile[ring][lane][0]);
+        }
+        if ((k + 2) * kTT <= min_ntok) {
+            run_tile<CHUNK, false>(nxt, h, (k + 1) * kTT, my_ntok, since_key, block_size, keys, key_pos);
+        } else {
+            run_tile<CHUNK, true>(nxt, h, (k + 1) * kTT, my_ntok, since_key, block_size, keys, key_pos);
         }
         lds_barrier();
     }
@@ -312,12 +442,15 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
         return KVCM_ERR_INVALID_ARG;
     }
     const dim3 grid(static_cast<uint32_t>((static_cast<int64_t>(R) + kReqs - 1) / kReqs));
+    // test hook: take the loader path that a workgroup spanning >= 4 GiB of tokens would take
+    const char *fg = std::getenv("KVCM_HASH_FORCE_GLOBAL_LOADS");
+    const int32_t force_global = (fg && fg[0] == '1') ? 1 : 0;
     if (block_size % 8 == 0) {
         hipLaunchKernelGGL((hash_tokens_kernel<TokT, 8>), grid, dim3(kThreads), 0, stream, d_tokens, d_token_offsets, R,
-                           block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets);
+                           block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global);
     } else {
         hipLaunchKernelGGL((hash_tokens_kernel<TokT, 1>), grid, dim3(kThreads), 0, stream, d_tokens, d_token_offsets, R,
-                           block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets);
+                           block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global);
     }
     return launch_status();
 }

@@ -70,6 +70,28 @@ def test_ragged_batch_and_seed(oracle):
         sync()
         assert (host(off, np.int64) == woff).all()
         assert (host(keys, np.int64) == want).all(), (bs, seed)
+    # int32 tokens, ragged (request starts at odd element offsets: 16-byte loads at 4-byte alignment)
+    flat32 = flat.astype(np.int32)
+    want, _ = oracle.hash_tokens(flat32, 16, token_offsets=toff)
+    keys, _ = _h().hash_tokens(dev(flat32), 16, token_offsets=dev(toff))
+    sync()
+    assert (host(keys, np.int64) == want).all()
+
+
+@pytest.mark.parametrize("dtype", [np.int64, np.int32])
+def test_general_loader_path(oracle, monkeypatch, dtype):
+    """The loader form used when a workgroup's requests span 4 GiB or more (32-bit buffer offsets cannot reach),
+    forced here through its test hook, on a ragged batch whose last request ends exactly at the end of the buffer."""
+    monkeypatch.setenv("KVCM_HASH_FORCE_GLOBAL_LOADS", "1")
+    rng = np.random.default_rng(17)
+    lens = [int(x) for x in rng.integers(0, 900, size=150)] + [64]
+    flat = rng.integers(-2**31, 2**31 - 1, size=sum(lens), dtype=np.int64).astype(dtype)
+    toff = np.zeros(len(lens) + 1, dtype=np.int64)
+    np.cumsum(lens, out=toff[1:])
+    want, woff = oracle.hash_tokens(flat, 16, token_offsets=toff)
+    keys, off = _h().hash_tokens(dev(flat), 16, token_offsets=dev(toff))
+    sync()
+    assert (host(keys, np.int64) == want).all()
 
 
 def test_config2_batch_prefix_property(oracle):
