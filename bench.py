@@ -125,6 +125,9 @@ def main():
     ap.add_argument("--pool-blocks", type=int, default=32768, help="blocks per layer in the paged pool")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--calibrate-copy-gib", type=float, default=0.0,
+                    help="also run one plain device-to-device copy of this many GiB after the timed region, so that a "
+                         "rocprofv3 --pmc run of this command holds a copy kernel of known size to scale counters by")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this path has no collectives and every box here has one GPU; "
@@ -185,6 +188,14 @@ def main():
     ms_gather = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
     ms_scatter = sum(e[2].elapsed_time(e[3]) for e in events) / args.steps
     ms_step = wall * 1e3 / args.steps
+
+    if args.calibrate_copy_gib > 0:
+        n = int(args.calibrate_copy_gib * 2**30)
+        src = staging.view(torch.uint8).reshape(-1)[:n]
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del dst
 
     verified = None
     if not args.no_verify:

@@ -6,16 +6,19 @@
 // launch shape does not: the reference runs 3 programs that walk all blocks serially because its staging
 // buffer sits behind PCIe, here staging is HBM and the device is filled.
 //
-// Work decomposition (gfx950, wave64):
-//   tile   = one (pool array p, work block b): T rows, contiguous in staging, `runs` contiguous runs in
-//            the pool. One wavefront moves one tile with 16-byte accesses, 8 loads in flight per lane
-//            before the first store.
-//   unit   = one work block b and a group of `tiles_per_wg` consecutive p: one workgroup of 4 waves.
-//            The block's run-start slots are read once per workgroup into LDS; the four waves then
-//            take p = first, first+4, ...
-//   The layer-major -> block-major transposition is only address arithmetic: a lane's 16 bytes go
-//   from pool_p + slot*row_bytes + off to staging + sb*block_stride + p*tile_stride + run*run_bytes + off
-//   through registers; nothing is reshaped in memory.
+// Work decomposition (gfx950, wave64), chosen by measurement on MI355X:
+//   A staging block is a run of 16-byte chunks, tile after tile ([P][T*row_bytes]). A workgroup of 1024
+//   threads (16 waves) takes one SPAN of 2048 consecutive chunks = 32 KiB of staging -- for the Llama-3-8B
+//   layout exactly one (layer, K/V, block) tile -- and every thread moves two chunks: two 16-byte loads in
+//   flight, then two 16-byte stores. The whole 32 KiB is therefore read and written in one short burst by
+//   one workgroup. HBM favours that: against one wavefront streaming a tile by itself (8 KiB per pass,
+//   the tile's rows trickling out over microseconds) the burst form moved 5.3 -> 5.85 TB/s on scatter and
+//   5.5 -> 6.0 TB/s on gather in a standalone sweep, because each 32 KiB pool chunk is written while its
+//   DRAM pages are still open instead of competing with 2000 other half-written chunks.
+//   The layer-major -> block-major transposition is only address arithmetic: a thread's 16 bytes go from
+//   pool_p + slot*row_bytes + off to staging + sb*block_stride + p*tile_stride + run*run_bytes + off through
+//   registers; nothing is reshaped in memory. Chunk -> (tile, run, offset) uses two multiply-shift divisions.
+//   All accesses carry the non-temporal hint: every byte is touched once.
 //
 // Roofline: HBM. Algorithmic bytes per tile = 2 * T * row_bytes (+ trailer), index bytes are negligible.
 #include "kvcm_internal.h"
@@ -27,13 +30,11 @@ namespace kvcm {
 namespace {
 
 #ifndef KVCM_COPY_THREADS
-#define KVCM_COPY_THREADS 256
+#define KVCM_COPY_THREADS 1024
 #endif
-#ifndef KVCM_COPY_UNROLL
-#define KVCM_COPY_UNROLL 8
+#ifndef KVCM_COPY_CHUNKS_PER_THREAD
+#define KVCM_COPY_CHUNKS_PER_THREAD 2
 #endif
-// Every byte is touched once, so loads and stores carry the non-temporal hint (streaming policy in L2):
-// measured +10 % on gather at the Llama-3-8B layout against plain accesses.
 #ifndef KVCM_COPY_NT_LOAD
 #define KVCM_COPY_NT_LOAD 1
 #endif
@@ -42,179 +43,218 @@ namespace {
 #endif
 
 constexpr int kThreads = KVCM_COPY_THREADS;
-constexpr int kWaves = kThreads / 64;
-constexpr int kMaxRuns = 2048;          // run-start slots of one work block staged in LDS (8 KiB)
-constexpr int kUnroll = KVCM_COPY_UNROLL;  // 16-byte accesses in flight per lane
+constexpr int kCPT = KVCM_COPY_CHUNKS_PER_THREAD;  // chunks per thread per span
+constexpr uint32_t kSpan = static_cast<uint32_t>(kThreads) * kCPT;
+
+// n / d for n < 2^31 as a multiply and a shift: mul = ceil(2^(31+L) / d), L = ceil(log2 d).
+struct FastDiv {
+    uint32_t mul;
+    uint32_t shift;
+};
+
+FastDiv make_fastdiv(uint32_t d) {
+    uint32_t L = 0;
+    while ((uint64_t{1} << L) < d) {
+        ++L;
+    }
+    const uint64_t pow = uint64_t{1} << (31 + L);
+    return FastDiv{static_cast<uint32_t>((pow + d - 1) / d), 31 + L};
+}
+
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, FastDiv f) {
+    return static_cast<uint32_t>((static_cast<uint64_t>(n) * f.mul) >> f.shift);
+}
 
 struct CopyArgs {
-    const void *const *ptr_table;
-    const void *const *trailer_table;
     unsigned char *staging;
-    const int32_t *run_start;
-    const int32_t *staging_idx;
-    const int32_t *trailer_idx;
     int64_t entry_stride;
     int64_t block_stride;
     int64_t tile_stride;
     int64_t row_bytes;
-    int64_t run_bytes;
-    int32_t P;
-    int32_t ptrs_per_entry;
-    int32_t runs;
+    int64_t tile_payload;  // T * row_bytes: where the trailer starts inside a staging tile
+    uint32_t ptrs_per_entry;
+    uint32_t runs;
     int32_t slot_limit;
     int32_t trailer_bytes;
-    int32_t tiles_per_wg;
-    uint32_t pgroups;
+    uint32_t chunks_per_run;
+    uint32_t chunks_per_tile;
+    uint32_t chunks_per_block;
+    uint32_t units_per_block;
     uint32_t n_units;
-    int32_t host_align;   // 16, 4 or 1: alignment shared by staging base, all strides and row_bytes
+    FastDiv div_tile;
+    FastDiv div_run;
+    FastDiv div_entry;
+    FastDiv div_units;
     int32_t xcd_remap;
 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-// 16 bytes at dword alignment: still one dwordx4 access (global memory accepts dword-aligned wide
-// accesses); used when a 4-byte trailer shifts every staging tile off the 16-byte grid.
+// 16 bytes at dword alignment: still ONE dwordx4 instruction (global memory takes dword-aligned wide accesses);
+// the alignment only tells the compiler what it may assume. A 4-byte trailer per tile shifts staging tiles off
+// the 16-byte grid, so the 16-byte path never promises more than dword alignment.
 typedef u32x4 u32x4_dword_aligned __attribute__((aligned(4)));
 
-// Access descriptors: the register type V and the pointer type P the memory access goes through.
-struct Acc16 {
-    using V = u32x4;
-    using P = u32x4;
-};
-struct Acc16U {
+template <int CS>
+struct Chunk;
+template <>
+struct Chunk<16> {
     using V = u32x4;
     using P = u32x4_dword_aligned;
 };
-struct Acc4 {
+template <>
+struct Chunk<4> {
     using V = uint32_t;
     using P = uint32_t;
 };
-struct Acc1 {
+template <>
+struct Chunk<1> {
     using V = uint8_t;
     using P = uint8_t;
 };
 
-// The access goes through A::P so that its alignment (not the register type's) is what the compiler assumes.
-template <typename A>
-__device__ __forceinline__ typename A::V load_chunk(const unsigned char *p) {
+// Pool rows and staging are device (or pinned host) memory: the accesses name the global address space, so the
+// compiler emits global_load / global_store rather than flat instructions for pointers it read from a table.
+#define KVCM_GLOBAL __attribute__((address_space(1)))
+
+template <int CS>
+__device__ __forceinline__ typename Chunk<CS>::V load_chunk(const unsigned char *p) {
+    using GP = const KVCM_GLOBAL typename Chunk<CS>::P *;
 #if KVCM_COPY_NT_LOAD
-    return __builtin_nontemporal_load(reinterpret_cast<const typename A::P *>(p));
+    return __builtin_nontemporal_load((GP)(p));
 #else
-    return *reinterpret_cast<const typename A::P *>(p);
+    return *(GP)(p);
 #endif
 }
 
-template <typename A>
-__device__ __forceinline__ void store_chunk(unsigned char *p, typename A::V v) {
+template <int CS>
+__device__ __forceinline__ void store_chunk(unsigned char *p, typename Chunk<CS>::V v) {
+    using GP = KVCM_GLOBAL typename Chunk<CS>::P *;
 #if KVCM_COPY_NT_STORE
-    __builtin_nontemporal_store(v, reinterpret_cast<typename A::P *>(p));
+    __builtin_nontemporal_store(v, (GP)(p));
 #else
-    *reinterpret_cast<typename A::P *>(p) = v;
+    *(GP)(p) = v;
 #endif
 }
 
-// Moves one tile. `runs_lds` holds the first slot of every run. Chunks (sizeof(V) bytes) are numbered
-// along the staging tile; chunk c belongs to run c / cpr at offset c % cpr. A lane visits chunks
-// lane, lane + 64, ... and keeps (run, offset) up to date incrementally, so the loop has no division.
-template <typename A, bool SCATTER>
-__device__ __forceinline__ void move_tile(unsigned char *pool, unsigned char *tile, const int32_t *runs_lds,
-                                          const CopyArgs &a, uint32_t lane) {
-    using V = typename A::V;
-    const uint32_t cpr = static_cast<uint32_t>(a.run_bytes / static_cast<int64_t>(sizeof(V)));
-    const uint32_t total = static_cast<uint32_t>(a.runs) * cpr;
-    const uint32_t step_r = 64u / cpr;
-    const uint32_t step_off = 64u - step_r * cpr;
-    const int64_t limit = a.slot_limit > 0 ? a.slot_limit : INT64_MAX;
-    uint32_t r = lane / cpr;
-    uint32_t off = lane - r * cpr;
-    for (uint32_t c0 = lane; c0 < total; c0 += 64u * kUnroll) {
-        V v[kUnroll];
-        unsigned char *pp[kUnroll];
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            pp[u] = nullptr;
-            if (c0 + 64u * u < total) {
-                const int64_t slot = runs_lds[r];
-                if (slot >= 0 && slot < limit) {
-                    pp[u] = pool + slot * a.row_bytes + static_cast<int64_t>(off) * sizeof(V);
-                }
-            }
-            off += step_off;
-            r += step_r;
-            if (off >= cpr) {
-                off -= cpr;
-                r += 1;
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            if (pp[u]) {
-                const unsigned char *sp = tile + static_cast<int64_t>(c0 + 64u * u) * sizeof(V);
-                v[u] = load_chunk<A>(SCATTER ? sp : pp[u]);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            if (pp[u]) {
-                unsigned char *sp = tile + static_cast<int64_t>(c0 + 64u * u) * sizeof(V);
-                store_chunk<A>(SCATTER ? pp[u] : sp, v[u]);
-            }
-        }
-    }
-}
+// CS = chunk size in bytes (16, 4 or 1), picked on the host from what it can see: staging address, strides,
+// row size. Pool base pointers live in device memory; a pool row that is not dword-aligned (CS > 1) is moved
+// byte by byte by the one thread that owns the chunk.
+//
+// UNI_TILE: every span lies inside one tile (chunks_per_tile is a multiple of the span), so the tile number, the
+// pool base pointer and the staging tile address are workgroup-uniform: scalar arithmetic and scalar loads.
+// UNI_RUN: every span also lies inside one run of consecutive slots (block-table fast path with runs of 32 KiB
+// or more), so the run's first slot is one scalar load as well and a thread's own work is two address adds.
+// Without them the same quantities are computed per thread and the index / pointer come through vector loads.
+template <int CS, bool SCATTER, bool UNI_TILE, bool UNI_RUN>
+__global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
+                                                             // read-only tables, never written by this kernel:
+                                                             // __restrict__ lets uniform reads become scalar loads
+                                                             const void *const *__restrict__ ptr_table,
+                                                             const void *const *__restrict__ trailer_table,
+                                                             const int32_t *__restrict__ run_start,
+                                                             const int32_t *__restrict__ staging_idx,
+                                                             const int32_t *__restrict__ trailer_idx) {
+    using V = typename Chunk<CS>::V;
 
-template <bool SCATTER>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))) void copy_tiles_kernel(const CopyArgs a) {
-    __shared__ int32_t s_runs[kMaxRuns];
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-
-    // Consecutive workgroup ids land on consecutive XCDs (8 per device, one L2 each). With the remap
-    // every XCD walks one contiguous eighth of the unit range instead of every eighth unit.
+    // Consecutive workgroup ids land on consecutive XCDs (8 per device, one L2 each). With the remap every XCD
+    // walks one contiguous eighth of the unit range instead of every eighth unit.
     uint32_t first = blockIdx.x;
     if (a.xcd_remap) {
         const uint32_t q = gridDim.x >> 3, rem = gridDim.x & 7u;
         const uint32_t xcd = blockIdx.x & 7u, idx = blockIdx.x >> 3;
         first = xcd * q + (xcd < rem ? xcd : rem) + idx;
     }
+    const int64_t limit = a.slot_limit > 0 ? a.slot_limit : INT64_MAX;
 
     for (uint32_t unit = first; unit < a.n_units; unit += gridDim.x) {
-        const uint32_t b = unit / a.pgroups;
-        const uint32_t pg = unit - b * a.pgroups;
-        __syncthreads();
-        for (int32_t i = threadIdx.x; i < a.runs; i += kThreads) {
-            s_runs[i] = a.run_start[static_cast<int64_t>(b) * a.runs + i];
-        }
-        __syncthreads();
-        const int64_t slot = a.staging_idx ? a.staging_idx[b] : static_cast<int64_t>(b);
-        unsigned char *block = a.staging + slot * a.block_stride;
-        const int32_t p_begin = static_cast<int32_t>(pg) * a.tiles_per_wg;
-        const int32_t p_end = min(a.P, p_begin + a.tiles_per_wg);
-        for (int32_t p = p_begin + static_cast<int32_t>(wave); p < p_end; p += kWaves) {
-            const int32_t entry = p / a.ptrs_per_entry;
-            const int32_t inner = p - entry * a.ptrs_per_entry;
-            unsigned char *pool = static_cast<unsigned char *>(const_cast<void *>(a.ptr_table[entry])) +
-                                  static_cast<int64_t>(inner) * a.entry_stride;
-            unsigned char *tile = block + static_cast<int64_t>(p) * a.tile_stride;
-            const uintptr_t pa = reinterpret_cast<uintptr_t>(pool);
-            if (a.host_align == 16 && (pa & 15u) == 0) {
-                move_tile<Acc16, SCATTER>(pool, tile, s_runs, a, lane);
-            } else if (a.host_align >= 4 && (pa & 3u) == 0 && (a.run_bytes & 15) == 0) {
-                move_tile<Acc16U, SCATTER>(pool, tile, s_runs, a, lane);
-            } else if (a.host_align >= 4 && (pa & 3u) == 0) {
-                move_tile<Acc4, SCATTER>(pool, tile, s_runs, a, lane);
-            } else {
-                move_tile<Acc1, SCATTER>(pool, tile, s_runs, a, lane);
-            }
-            if (a.trailer_bytes > 0) {
-                unsigned char *tr = static_cast<unsigned char *>(const_cast<void *>(a.trailer_table[p])) +
-                                    static_cast<int64_t>(a.trailer_idx[b]) * a.trailer_bytes;
-                unsigned char *st = tile + static_cast<int64_t>(a.runs) * a.run_bytes;
-                for (int32_t i = lane; i < a.trailer_bytes; i += 64) {
-                    if (SCATTER) {
-                        tr[i] = st[i];
-                    } else {
-                        st[i] = tr[i];
+        const uint32_t b = fast_div(unit, a.div_units);
+        const uint32_t span = unit - b * a.units_per_block;
+        const int32_t *runs_b = run_start + static_cast<int64_t>(b) * a.runs;
+        // workgroup-uniform part: the three table reads below are independent scalar loads in the UNI_* forms
+        const uint32_t g_first = span * kSpan;
+        const uint32_t p_first = fast_div(g_first, a.div_tile);
+        const uint32_t cc_first = g_first - p_first * a.chunks_per_tile;
+        const uint32_t r_first = fast_div(cc_first, a.div_run);
+        const uint32_t entry_first = fast_div(p_first, a.div_entry);
+        const int64_t slot_first = UNI_RUN ? runs_b[r_first] : 0;
+        const void *pool_first = UNI_TILE ? ptr_table[entry_first] : nullptr;
+        const int64_t slot_b = staging_idx ? staging_idx[b] : static_cast<int64_t>(b);
+        unsigned char *block = a.staging + slot_b * a.block_stride;
+
+        V v[kCPT];
+        unsigned char *pp[kCPT];
+        unsigned char *sp[kCPT];
+#pragma unroll
+        for (int u = 0; u < kCPT; ++u) {
+            const uint32_t in_span = threadIdx.x + static_cast<uint32_t>(u) * kThreads;
+            const uint32_t g = g_first + in_span;
+            pp[u] = nullptr;
+            sp[u] = nullptr;
+            if (g < a.chunks_per_block) {
+                const uint32_t p = UNI_TILE ? p_first : fast_div(g, a.div_tile);
+                const uint32_t cc = UNI_TILE ? cc_first + in_span : g - p * a.chunks_per_tile;
+                const uint32_t r = UNI_RUN ? r_first : fast_div(cc, a.div_run);
+                const uint32_t off = cc - r * a.chunks_per_run;
+                const int64_t slot = UNI_RUN ? slot_first : static_cast<int64_t>(runs_b[r]);
+                unsigned char *tile = block + static_cast<int64_t>(p) * a.tile_stride;
+                if (slot >= 0 && slot < limit) {
+                    const uint32_t entry = UNI_TILE ? entry_first : fast_div(p, a.div_entry);
+                    const uint32_t inner = p - entry * a.ptrs_per_entry;
+                    const void *base = UNI_TILE ? pool_first : ptr_table[entry];
+                    unsigned char *pool = static_cast<unsigned char *>(const_cast<void *>(base)) +
+                                          static_cast<int64_t>(inner) * a.entry_stride;
+                    pp[u] = pool + slot * a.row_bytes + static_cast<int64_t>(off) * CS;
+                    sp[u] = tile + static_cast<int64_t>(cc) * CS;
+                }
+                if (a.trailer_bytes > 0 && cc == 0) {
+                    // the thread that owns a tile's first chunk also moves the tile's trailer
+                    unsigned char *tr = static_cast<unsigned char *>(const_cast<void *>(trailer_table[p])) +
+                                        static_cast<int64_t>(trailer_idx[b]) * a.trailer_bytes;
+                    unsigned char *st = tile + a.tile_payload;
+                    for (int32_t i = 0; i < a.trailer_bytes; ++i) {
+                        if (SCATTER) {
+                            tr[i] = st[i];
+                        } else {
+                            st[i] = tr[i];
+                        }
                     }
+                }
+            }
+        }
+        // Common case: every chunk of this thread is live and dword-aligned. One straight-line block -- all loads
+        // back to back, then all stores -- so that no store waits for an earlier store's acknowledgement.
+        bool all_fast = true;
+#pragma unroll
+        for (int u = 0; u < kCPT; ++u) {
+            all_fast = all_fast && pp[u] && (CS == 1 || (reinterpret_cast<uintptr_t>(pp[u]) & 3u) == 0);
+        }
+        if (all_fast) {
+#pragma unroll
+            for (int u = 0; u < kCPT; ++u) {
+                v[u] = load_chunk<CS>(SCATTER ? sp[u] : pp[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < kCPT; ++u) {
+                store_chunk<CS>(SCATTER ? pp[u] : sp[u], v[u]);
+            }
+        } else {
+            // Ragged end of a block, skipped rows, or a pool row that is not dword-aligned (never the case for an
+            // engine's own allocations): chunk by chunk, bytes where the alignment demands it.
+#pragma unroll
+            for (int u = 0; u < kCPT; ++u) {
+                if (!pp[u]) {
+                    continue;
+                }
+                if (CS > 1 && (reinterpret_cast<uintptr_t>(pp[u]) & 3u) != 0) {
+                    for (int i = 0; i < CS; ++i) {
+                        if (SCATTER) {
+                            pp[u][i] = sp[u][i];
+                        } else {
+                            sp[u][i] = pp[u][i];
+                        }
+                    }
+                } else {
+                    store_chunk<CS>(SCATTER ? pp[u] : sp[u], load_chunk<CS>(SCATTER ? sp[u] : pp[u]));
                 }
             }
         }
@@ -258,6 +298,17 @@ int32_t align_class(uint64_t bits) {
     return 1;
 }
 
+template <int CS, bool UNI_TILE, bool UNI_RUN>
+void launch_span(const CopyArgs &a, const kvcm_copy_desc *d, bool scatter, uint32_t grid, hipStream_t stream) {
+    if (scatter) {
+        hipLaunchKernelGGL((copy_span_kernel<CS, true, UNI_TILE, UNI_RUN>), dim3(grid), dim3(kThreads), 0, stream, a,
+                           d->d_ptr_table, d->d_trailer_ptr_table, d->d_run_start, d->d_staging_idx, d->d_trailer_idx);
+    } else {
+        hipLaunchKernelGGL((copy_span_kernel<CS, false, UNI_TILE, UNI_RUN>), dim3(grid), dim3(kThreads), 0, stream, a,
+                           d->d_ptr_table, d->d_trailer_ptr_table, d->d_run_start, d->d_staging_idx, d->d_trailer_idx);
+    }
+}
+
 int32_t launch_copy(const kvcm_copy_desc *d, bool scatter, hipStream_t stream) {
     if (!d) {
         return KVCM_ERR_INVALID_ARG;
@@ -283,62 +334,60 @@ int32_t launch_copy(const kvcm_copy_desc *d, bool scatter, hipStream_t stream) {
     if (d->trailer_bytes > 0 && (!d->d_trailer_ptr_table || !d->d_trailer_idx)) {
         return KVCM_ERR_INVALID_ARG;
     }
-    const int32_t runs = d->T / d->run_tokens;
-    if (runs > kMaxRuns || payload >= (int64_t{1} << 31)) {
+    // one staging block must be addressable with 31-bit chunk numbers in every chunk size
+    if (payload * d->P >= (int64_t{1} << 31)) {
         return KVCM_ERR_TOO_LARGE;
     }
 
     CopyArgs a{};
-    a.ptr_table = d->d_ptr_table;
-    a.trailer_table = d->d_trailer_ptr_table;
     a.staging = static_cast<unsigned char *>(d->d_staging);
-    a.run_start = d->d_run_start;
-    a.staging_idx = d->d_staging_idx;
-    a.trailer_idx = d->d_trailer_idx;
     a.entry_stride = d->entry_stride_bytes;
     a.block_stride = d->staging_block_stride_bytes;
     a.tile_stride = d->staging_tile_stride_bytes;
     a.row_bytes = d->row_bytes;
-    a.run_bytes = static_cast<int64_t>(d->run_tokens) * d->row_bytes;
-    a.P = d->P;
-    a.ptrs_per_entry = d->ptrs_per_entry;
-    a.runs = runs;
+    a.tile_payload = payload;
+    a.ptrs_per_entry = static_cast<uint32_t>(d->ptrs_per_entry);
+    a.runs = static_cast<uint32_t>(d->T / d->run_tokens);
     a.slot_limit = d->slot_limit;
     a.trailer_bytes = d->trailer_bytes;
-    a.host_align = align_class(reinterpret_cast<uint64_t>(d->d_staging) | static_cast<uint64_t>(a.block_stride) |
-                               static_cast<uint64_t>(a.tile_stride) | static_cast<uint64_t>(a.row_bytes) |
-                               static_cast<uint64_t>(a.entry_stride));
 
-    // Tiles per workgroup: one per wave when tiles are large; more for small tiles so that a workgroup
-    // moves at least 64 KiB, as long as enough workgroups remain to fill the device.
-    const int cus = device_cu_count();
-    int32_t tpw = kWaves;
-    while (tpw < d->P && payload * tpw < 65536 &&
-           static_cast<int64_t>(d->B) * ((d->P + 2 * tpw - 1) / (2 * tpw)) >= static_cast<int64_t>(cus) * 8) {
-        tpw *= 2;
-    }
-    tpw = env_int("KVCM_COPY_TILES_PER_WG", tpw);
-    a.tiles_per_wg = tpw;
-    a.pgroups = static_cast<uint32_t>((d->P + tpw - 1) / tpw);
-    const int64_t units = static_cast<int64_t>(d->B) * a.pgroups;
+    const int64_t run_bytes = static_cast<int64_t>(d->run_tokens) * d->row_bytes;
+    const int32_t cls = align_class(reinterpret_cast<uint64_t>(d->d_staging) | static_cast<uint64_t>(a.block_stride) |
+                                    static_cast<uint64_t>(a.tile_stride) | static_cast<uint64_t>(a.row_bytes) |
+                                    static_cast<uint64_t>(a.entry_stride));
+    const int cs = (cls >= 4 && (run_bytes & 15) == 0) ? 16 : (cls >= 4 ? 4 : 1);
+    a.chunks_per_run = static_cast<uint32_t>(run_bytes / cs);
+    a.chunks_per_tile = a.runs * a.chunks_per_run;
+    a.chunks_per_block = a.chunks_per_tile * static_cast<uint32_t>(d->P);
+    a.units_per_block = (a.chunks_per_block + kSpan - 1) / kSpan;
+    const int64_t units = static_cast<int64_t>(d->B) * a.units_per_block;
     if (units >= (int64_t{1} << 31)) {
         return KVCM_ERR_TOO_LARGE;
     }
     a.n_units = static_cast<uint32_t>(units);
+    a.div_tile = make_fastdiv(a.chunks_per_tile);
+    a.div_run = make_fastdiv(a.chunks_per_run);
+    a.div_entry = make_fastdiv(a.ptrs_per_entry);
+    a.div_units = make_fastdiv(a.units_per_block);
     a.xcd_remap = env_int("KVCM_COPY_XCD_REMAP", 1);
 
     int64_t grid = units;
-    const int per_cu = env_int("KVCM_COPY_WG_PER_CU", 0);
-    if (per_cu > 0) {
-        grid = std::min<int64_t>(grid, static_cast<int64_t>(cus) * per_cu);
-    }
     if (d->max_workgroups > 0) {
         grid = std::min<int64_t>(grid, d->max_workgroups);
     }
-    if (scatter) {
-        hipLaunchKernelGGL(copy_tiles_kernel<true>, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0, stream, a);
+    const bool uni_tile = a.chunks_per_tile % kSpan == 0;
+    const bool uni_run = uni_tile && a.chunks_per_run % kSpan == 0;
+    const uint32_t g32 = static_cast<uint32_t>(grid);
+    if (cs == 16 && uni_run) {
+        launch_span<16, true, true>(a, d, scatter, g32, stream);
+    } else if (cs == 16 && uni_tile) {
+        launch_span<16, true, false>(a, d, scatter, g32, stream);
+    } else if (cs == 16) {
+        launch_span<16, false, false>(a, d, scatter, g32, stream);
+    } else if (cs == 4) {
+        launch_span<4, false, false>(a, d, scatter, g32, stream);
     } else {
-        hipLaunchKernelGGL(copy_tiles_kernel<false>, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0, stream, a);
+        launch_span<1, false, false>(a, d, scatter, g32, stream);
     }
     return launch_status();
 }

@@ -51,7 +51,8 @@ def test_argument_validation_needs_no_device():
     assert L.kvcm_hip_batch_gather(p, 2, p, 64, p, None, 1, 16, 64, 0, None) == _lib.ERR_INVALID_ARG  # slot too small
     assert L.kvcm_hip_batch_gather(None, 2, p, 2 * 16 * 64, p, None, 1, 16, 64, 0, None) == _lib.ERR_INVALID_ARG
     assert L.kvcm_hip_paged_gather(p, 2, p, 2 * 16 * 64, p, 3, None, 1, 16, 64, 0, None) == _lib.ERR_INVALID_ARG
-    assert L.kvcm_hip_batch_scatter(p, 2, p, 2 * 4096 * 64, p, None, 1, 4096, 64, 0, None) == _lib.ERR_TOO_LARGE
+    # a staging block of 2 GiB or more cannot be numbered with 31-bit chunk indices
+    assert L.kvcm_hip_batch_scatter(p, 2, p, 1 << 34, p, None, 1, 1 << 20, 1 << 12, 0, None) == _lib.ERR_TOO_LARGE
     # nothing to do is not an error
     assert L.kvcm_hip_batch_gather(p, 2, p, 2 * 16 * 64, p, None, 0, 16, 64, 0, None) == _lib.OK
     assert L.kvcm_hip_hash_tokens(p, p, 0, 16, 0, p, None, None) == _lib.OK
