@@ -7,18 +7,26 @@
 // buffer sits behind PCIe, here staging is HBM and the device is filled.
 //
 // Work decomposition (gfx950, wave64), chosen by measurement on MI355X:
-//   A staging block is a run of 16-byte chunks, tile after tile ([P][T*row_bytes]). A workgroup of 1024
-//   threads (16 waves) takes one SPAN of 2048 consecutive chunks = 32 KiB of staging -- for the Llama-3-8B
-//   layout exactly one (layer, K/V, block) tile -- and every thread moves two chunks: two 16-byte loads in
-//   flight, then two 16-byte stores. The whole 32 KiB is therefore read and written in one short burst by
-//   one workgroup. HBM favours that: against one wavefront streaming a tile by itself (8 KiB per pass,
-//   the tile's rows trickling out over microseconds) the burst form moved 5.3 -> 5.85 TB/s on scatter and
-//   5.5 -> 6.0 TB/s on gather in a standalone sweep, because each 32 KiB pool chunk is written while its
-//   DRAM pages are still open instead of competing with 2000 other half-written chunks.
+//   A staging block is a run of 16-byte chunks, tile after tile ([P][T*row_bytes]). A workgroup of 256 threads
+//   (4 waves) takes one SPAN of 256 consecutive chunks = 4 KiB of staging and every thread moves exactly one
+//   chunk: one 16-byte load, one 16-byte store, done. There is no loop and nothing to unroll; memory-level
+//   parallelism comes from the ~32 resident waves per CU, each with one access in flight, and from the
+//   dispatcher replacing finished workgroups. For the Llama-3-8B layout a (layer, K/V, block) tile is 8 spans.
+//   Measured at that layout (12 416 blocks, 2 x 24.25 GiB per launch, % of the 8 TB/s HBM peak):
+//       one wavefront streams a whole 32 KiB tile, 8 loads in flight per lane      gather 74 %   scatter 68 %
+//       1024 threads x 2 chunks, one 32 KiB tile per workgroup                      gather 75 %   scatter 74 %
+//       256 threads x 1 chunk (this kernel)                                         gather 79 %   scatter 77 %
+//   The fine-grained form wins because each 4 KiB piece of a pool block is read or written in one short burst
+//   while its DRAM pages are open, instead of trickling out of a long-lived wave that shares the memory
+//   controllers with 2000 other half-finished tiles; scattered 32 KiB writes gain the most.
+//   Workgroup ids are dealt round-robin to the 8 XCDs; the kernel renumbers them so that every XCD walks one
+//   contiguous eighth of the span range (+6 % against leaving consecutive 4 KiB spans on different XCDs).
 //   The layer-major -> block-major transposition is only address arithmetic: a thread's 16 bytes go from
 //   pool_p + slot*row_bytes + off to staging + sb*block_stride + p*tile_stride + run*run_bytes + off through
-//   registers; nothing is reshaped in memory. Chunk -> (tile, run, offset) uses two multiply-shift divisions.
-//   All accesses carry the non-temporal hint: every byte is touched once.
+//   registers; nothing is reshaped in memory. When a span lies inside one tile (and one run) the tile number,
+//   pool pointer and slot are workgroup-uniform: scalar arithmetic and scalar loads, and a thread's own work is
+//   two address adds. Otherwise chunk -> (tile, run, offset) is two multiply-shift divisions per thread.
+//   All accesses carry the non-temporal hint: every byte is touched once (+4 % gather against plain accesses).
 //
 // Roofline: HBM. Algorithmic bytes per tile = 2 * T * row_bytes (+ trailer), index bytes are negligible.
 #include "kvcm_internal.h"
@@ -30,10 +38,10 @@ namespace kvcm {
 namespace {
 
 #ifndef KVCM_COPY_THREADS
-#define KVCM_COPY_THREADS 1024
+#define KVCM_COPY_THREADS 256
 #endif
 #ifndef KVCM_COPY_CHUNKS_PER_THREAD
-#define KVCM_COPY_CHUNKS_PER_THREAD 2
+#define KVCM_COPY_CHUNKS_PER_THREAD 1
 #endif
 #ifndef KVCM_COPY_NT_LOAD
 #define KVCM_COPY_NT_LOAD 1
@@ -142,8 +150,8 @@ __device__ __forceinline__ void store_chunk(unsigned char *p, typename Chunk<CS>
 //
 // UNI_TILE: every span lies inside one tile (chunks_per_tile is a multiple of the span), so the tile number, the
 // pool base pointer and the staging tile address are workgroup-uniform: scalar arithmetic and scalar loads.
-// UNI_RUN: every span also lies inside one run of consecutive slots (block-table fast path with runs of 32 KiB
-// or more), so the run's first slot is one scalar load as well and a thread's own work is two address adds.
+// UNI_RUN: every span also lies inside one run of consecutive slots (block-table fast path, or rows of 4 KiB
+// and more), so the run's first slot is one scalar load as well and a thread's own work is two address adds.
 // Without them the same quantities are computed per thread and the index / pointer come through vector loads.
 template <int CS, bool SCATTER, bool UNI_TILE, bool UNI_RUN>
 __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
@@ -222,7 +230,8 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
             }
         }
         // Common case: every chunk of this thread is live and dword-aligned. One straight-line block -- all loads
-        // back to back, then all stores -- so that no store waits for an earlier store's acknowledgement.
+        // back to back, then all stores -- so that no store waits for an earlier store's acknowledgement (matters
+        // when the kernel is built with more than one chunk per thread).
         bool all_fast = true;
 #pragma unroll
         for (int u = 0; u < kCPT; ++u) {
