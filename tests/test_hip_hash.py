@@ -106,6 +106,15 @@ def test_config2_batch_prefix_property(oracle):
     assert len(np.unique(k[:, 128])) == 64 and len(np.unique(k[32:, 0])) == 32
 
 
+@pytest.mark.parametrize("R,L,bs,vocab", [(32, 16384, 64, 152064), (128, 8192, 128, 129280)])
+def test_config3_and_config4_batches(oracle, R, L, bs, vocab):
+    tok = cases.tokens(R, L, vocab, shared_rows=R // 2, shared_len=(L * 3 // 4 // bs) * bs, seed=0)
+    keys, _ = _h().hash_tokens(dev(tok), bs)
+    sync()
+    want, _ = oracle.hash_tokens(tok, bs, threads=8)
+    assert (host(keys, np.int64) == want).all()
+
+
 def test_config5_many_requests(oracle):
     tok = cases.tokens(1024, 1024, 152064, seed=0)
     keys, _ = _h().hash_tokens(dev(tok), 16)
