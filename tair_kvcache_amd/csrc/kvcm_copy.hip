@@ -150,10 +150,15 @@ __device__ __forceinline__ void store_chunk(unsigned char *p, typename Chunk<CS>
 //
 // UNI_TILE: every span lies inside one tile (chunks_per_tile is a multiple of the span), so the tile number, the
 // pool base pointer and the staging tile address are workgroup-uniform: scalar arithmetic and scalar loads.
-// UNI_RUN: every span also lies inside one run of consecutive slots (block-table fast path, or rows of 4 KiB
-// and more), so the run's first slot is one scalar load as well and a thread's own work is two address adds.
-// Without them the same quantities are computed per thread and the index / pointer come through vector loads.
-template <int CS, bool SCATTER, bool UNI_TILE, bool UNI_RUN>
+// RUN = how widely a run of consecutive slots is shared (needs UNI_TILE):
+//   kRunPerGroup  every span lies inside one run (block-table fast path, or rows of 4 KiB and more): the run's
+//                 first slot is one scalar load per workgroup and a thread's own work is two address adds;
+//   kRunPerWave   a run is a whole number of wavefronts' worth of chunks (rows of 1 KiB and more): the slot is a
+//                 scalar load per wave;
+//   kRunPerThread anything else: the run number is a multiply-shift division per thread and the slot a vector load.
+enum RunMode { kRunPerThread = 0, kRunPerWave = 1, kRunPerGroup = 2 };
+
+template <int CS, bool SCATTER, bool UNI_TILE, int RUN>
 __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
                                                              // read-only tables, never written by this kernel:
                                                              // __restrict__ lets uniform reads become scalar loads
@@ -184,7 +189,14 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
         const uint32_t cc_first = g_first - p_first * a.chunks_per_tile;
         const uint32_t r_first = fast_div(cc_first, a.div_run);
         const uint32_t entry_first = fast_div(p_first, a.div_entry);
-        const int64_t slot_first = UNI_RUN ? runs_b[r_first] : 0;
+        int64_t slot_shared = 0;
+        uint32_t r_shared = r_first;
+        if (RUN == kRunPerGroup) {
+            slot_shared = runs_b[r_first];
+        } else if (RUN == kRunPerWave) {
+            r_shared = __builtin_amdgcn_readfirstlane(fast_div(cc_first + (threadIdx.x & ~63u), a.div_run));
+            slot_shared = runs_b[r_shared];
+        }
         const void *pool_first = UNI_TILE ? ptr_table[entry_first] : nullptr;
         const int64_t slot_b = staging_idx ? staging_idx[b] : static_cast<int64_t>(b);
         unsigned char *block = a.staging + slot_b * a.block_stride;
@@ -201,9 +213,9 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
             if (g < a.chunks_per_block) {
                 const uint32_t p = UNI_TILE ? p_first : fast_div(g, a.div_tile);
                 const uint32_t cc = UNI_TILE ? cc_first + in_span : g - p * a.chunks_per_tile;
-                const uint32_t r = UNI_RUN ? r_first : fast_div(cc, a.div_run);
+                const uint32_t r = RUN != kRunPerThread ? r_shared : fast_div(cc, a.div_run);
                 const uint32_t off = cc - r * a.chunks_per_run;
-                const int64_t slot = UNI_RUN ? slot_first : static_cast<int64_t>(runs_b[r]);
+                const int64_t slot = RUN != kRunPerThread ? slot_shared : static_cast<int64_t>(runs_b[r]);
                 unsigned char *tile = block + static_cast<int64_t>(p) * a.tile_stride;
                 if (slot >= 0 && slot < limit) {
                     const uint32_t entry = UNI_TILE ? entry_first : fast_div(p, a.div_entry);
@@ -307,13 +319,13 @@ int32_t align_class(uint64_t bits) {
     return 1;
 }
 
-template <int CS, bool UNI_TILE, bool UNI_RUN>
+template <int CS, bool UNI_TILE, int RUN>
 void launch_span(const CopyArgs &a, const kvcm_copy_desc *d, bool scatter, uint32_t grid, hipStream_t stream) {
     if (scatter) {
-        hipLaunchKernelGGL((copy_span_kernel<CS, true, UNI_TILE, UNI_RUN>), dim3(grid), dim3(kThreads), 0, stream, a,
+        hipLaunchKernelGGL((copy_span_kernel<CS, true, UNI_TILE, RUN>), dim3(grid), dim3(kThreads), 0, stream, a,
                            d->d_ptr_table, d->d_trailer_ptr_table, d->d_run_start, d->d_staging_idx, d->d_trailer_idx);
     } else {
-        hipLaunchKernelGGL((copy_span_kernel<CS, false, UNI_TILE, UNI_RUN>), dim3(grid), dim3(kThreads), 0, stream, a,
+        hipLaunchKernelGGL((copy_span_kernel<CS, false, UNI_TILE, RUN>), dim3(grid), dim3(kThreads), 0, stream, a,
                            d->d_ptr_table, d->d_trailer_ptr_table, d->d_run_start, d->d_staging_idx, d->d_trailer_idx);
     }
 }
@@ -385,18 +397,19 @@ int32_t launch_copy(const kvcm_copy_desc *d, bool scatter, hipStream_t stream) {
         grid = std::min<int64_t>(grid, d->max_workgroups);
     }
     const bool uni_tile = a.chunks_per_tile % kSpan == 0;
-    const bool uni_run = uni_tile && a.chunks_per_run % kSpan == 0;
     const uint32_t g32 = static_cast<uint32_t>(grid);
-    if (cs == 16 && uni_run) {
-        launch_span<16, true, true>(a, d, scatter, g32, stream);
+    if (cs == 16 && uni_tile && a.chunks_per_run % kSpan == 0) {
+        launch_span<16, true, kRunPerGroup>(a, d, scatter, g32, stream);
+    } else if (cs == 16 && uni_tile && a.chunks_per_run % 64 == 0) {
+        launch_span<16, true, kRunPerWave>(a, d, scatter, g32, stream);
     } else if (cs == 16 && uni_tile) {
-        launch_span<16, true, false>(a, d, scatter, g32, stream);
+        launch_span<16, true, kRunPerThread>(a, d, scatter, g32, stream);
     } else if (cs == 16) {
-        launch_span<16, false, false>(a, d, scatter, g32, stream);
+        launch_span<16, false, kRunPerThread>(a, d, scatter, g32, stream);
     } else if (cs == 4) {
-        launch_span<4, false, false>(a, d, scatter, g32, stream);
+        launch_span<4, false, kRunPerThread>(a, d, scatter, g32, stream);
     } else {
-        launch_span<1, false, false>(a, d, scatter, g32, stream);
+        launch_span<1, false, kRunPerThread>(a, d, scatter, g32, stream);
     }
     return launch_status();
 }
