@@ -30,7 +30,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # from inside this process, so the figures are carried here and reported only for the workload they were taken on.
 MEASURED_TRAFFIC = {"unique_blocks": 12416, "gather": 52079641388, "scatter": 52076996342}
 
-# Llama-3-8B KV layout (BASELINE.json configs[1])
+# Llama-3-8B KV layout: the configuration the headline metric is quoted on
 LAYERS, KV_HEADS, HEAD_DIM, ITEMSIZE = 32, 8, 128, 2
 T = 16
 REQUESTS, TOKENS_PER_REQ, VOCAB = 64, 4096, 128256

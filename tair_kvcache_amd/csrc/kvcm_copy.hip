@@ -31,7 +31,6 @@
 // Roofline: HBM. Algorithmic bytes per tile = 2 * T * row_bytes (+ trailer), index bytes are negligible.
 #include "kvcm_internal.h"
 
-#include <atomic>
 #include <cstdlib>
 
 namespace kvcm {
@@ -437,24 +436,6 @@ kvcm_copy_desc flat_desc(const void *const *d_ptr_table, int32_t P, void *d_stag
 }
 
 }  // namespace
-
-int device_cu_count() {
-    static std::atomic<int> cache[64];
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
-        return 256;
-    }
-    int v = cache[dev].load(std::memory_order_relaxed);
-    if (v == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
-            n = 256;
-        }
-        cache[dev].store(n, std::memory_order_relaxed);
-        v = n;
-    }
-    return v;
-}
 
 }  // namespace kvcm
 

@@ -10,9 +10,6 @@ namespace kvcm {
 
 constexpr uint64_t kGolden = 0x9e3779b97f4a7c15ULL;
 
-// Compute units of the current device (cached per device; immutable after the first query).
-int device_cu_count();
-
 inline int32_t launch_status() {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? KVCM_OK : static_cast<int32_t>(e);

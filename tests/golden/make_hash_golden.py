@@ -22,7 +22,7 @@ from oracle import oracle as O  # noqa: E402
 
 
 def c1_tokens():
-    """BASELINE config 1 tokens: 4 requests x 512, uniform in [0,151936), first 256 shared. Seed 0."""
+    """Tokens of the smallest benchmark configuration: 4 requests x 512, uniform in [0,151936), first 256 shared. Seed 0."""
     rng = np.random.default_rng(0)
     tok = rng.integers(0, 151936, size=(4, 512), dtype=np.int64)
     tok[:, :256] = tok[0, :256]
