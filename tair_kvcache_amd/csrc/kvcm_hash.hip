@@ -6,16 +6,17 @@
 // + and ^, so a request is a serial chain of len dependent steps; the parallelism is across requests.
 //
 // Design (gfx950, wave64): a workgroup owns 64 requests and is role-split.
-//   wave 0      "chain wave": lane = request. Keeps the state in VGPRs and does nothing but the
-//               recurrence, reading pre-added terms a = v + C from LDS (one ds_read_b128 per 2 steps).
-//               A single wave issues about one instruction per 4 cycles, so every instruction removed
-//               from this wave shortens the critical path of all 64 chains.
-//   waves 1..3  "loader waves": stream the 64 requests' tokens from HBM in [64 requests x 32 tokens]
-//               tiles with coalesced 256-byte row segments, add C, and write them transposed into a
-//               3-deep LDS ring. Each loader wave owns every third tile and keeps its global loads in
-//               flight for about three tile periods, so HBM latency stays off the chain.
+//   wave 0      "chain wave": lane = request. Keeps the state in VGPRs and does nothing but the recurrence,
+//               reading pre-added terms a = v + C from LDS (one ds_read_b128 per 2 steps, prefetched a whole
+//               tile ahead into a second register set). A single wave issues about one instruction per 4.8
+//               cycles whether or not it depends on the previous one (measured), so every instruction removed
+//               from this wave shortens the critical path of all 64 chains: the step is 6 instructions.
+//   waves 1..3  "loader waves": stream the 64 requests' tokens from HBM in [64 requests x 64 tokens] tiles with
+//               16-byte buffer loads (512-byte row segments), add C, and write them transposed into a 3-slot LDS
+//               ring. Each loader wave owns every third tile and keeps its loads in flight for about three
+//               tile periods, so HBM latency stays off the chain.
 // Roofline: HBM for many requests (8*block_size + 8 bytes per key); for few requests the bound is the
-// dependent-instruction latency of the chain, which no amount of bandwidth removes.
+// instruction issue rate of the chain wave, which no amount of bandwidth removes.
 #include "kvcm_internal.h"
 
 #include <cstdlib>
@@ -23,17 +24,42 @@
 namespace kvcm {
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kReqs = 64;    // requests per workgroup = lanes of the chain wave
-constexpr int kTT = 32;      // tokens per request per tile
-constexpr int kRing = 3;     // LDS tiles in the ring
-constexpr int kPad = 2;      // keeps rows 16-byte aligned (b128 reads) and spreads banks
-constexpr int kLoaders = 3;  // loader waves
+#ifndef KVCM_HASH_LOADERS
+#define KVCM_HASH_LOADERS 3
+#endif
+#ifndef KVCM_HASH_TILE_TOKENS
+#define KVCM_HASH_TILE_TOKENS 64
+#endif
+
+constexpr int kLoaders = KVCM_HASH_LOADERS;   // loader waves
+constexpr int kThreads = 64 * (1 + kLoaders);
+constexpr int kReqs = 64;                     // requests per workgroup = lanes of the chain wave
+constexpr int kTT = KVCM_HASH_TILE_TOKENS;    // tokens per request per tile
+constexpr int kRing = kLoaders;               // LDS tiles in the ring: loader lw always fills slot lw
+constexpr int kPad = 2;                       // keeps rows 16-byte aligned (b128 reads) and spreads banks
 constexpr int kPerLane = kReqs * kTT / 64;  // tile elements per loader lane
 
 // Workgroup barrier that waits only for this wave's LDS traffic. __syncthreads() would also drain the
 // loader waves' outstanding global loads, which must stay in flight across barriers.
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// Spelled with builtins so that the compiler's own wait-count bookkeeping sees the LDS wait: after it the chain
+// wave's prefetched tile counts as arrived and its steps run without further waits.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0); vmcnt and expcnt left at their maxima
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// One step of the recurrence with the token term pre-added (a = v + C): h ^= a + (h << 12) + sar(h, 32).
+// Six single-issue VALU instructions: v_lshlrev_b64, v_ashrrev_i64, 2 x v_lshl_add_u64, 2 x v_xor_b32. The
+// arithmetic shift is written as the 64-bit instruction on purpose: left to itself the compiler splits sar(h, 32)
+// into v_ashrrev_i32 + v_mov_b32 (the pair {hi, sign} must be rebuilt in an even-aligned register pair), one
+// instruction more, and on a wave that is bound by instruction issue every instruction is 1/7 of the run time.
+__device__ __forceinline__ uint64_t chain_step(uint64_t h, uint64_t a) {
+    uint64_t sar;
+    asm("v_ashrrev_i64 %0, 32, %1" : "=v"(sar) : "v"(h));
+    return h ^ (a + (h << 12) + sar);
+}
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
@@ -177,7 +203,7 @@ __device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_
         if (active) {
 #pragma unroll
             for (int s = c; s < c + CHUNK; ++s) {
-                h = hash_step_preadded(h, (s & 1) ? a[s / 2].y : a[s / 2].x);
+                h = chain_step(h, (s & 1) ? a[s / 2].y : a[s / 2].x);
             }
         }
         since_key += CHUNK;
@@ -238,6 +264,11 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         max_ntok = hi_other > max_ntok ? hi_other : max_ntok;
         min_ntok = lo_other < min_ntok ? lo_other : min_ntok;
     }
+    // the reductions left the same value in every lane; say so, and loop control becomes scalar
+    max_ntok = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(max_ntok >> 32))) << 32) |
+               __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(max_ntok));
+    min_ntok = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(min_ntok >> 32))) << 32) |
+               __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(min_ntok));
     const int64_t ntiles = (max_ntok + kTT - 1) / kTT;  // uniform over the workgroup
     if (ntiles == 0) {
         return;
@@ -265,9 +296,8 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     }
 
     // -------------------------------------------------------------------- chain wave
-    // A single wave issues one VALU instruction per ~4.8 cycles whether or not it depends on the previous
-    // one (measured), so the step costs its instruction count: the compiler's 7 (v_lshlrev_b64, v_ashrrev_i32,
-    // v_mov, 2 x v_lshl_add_u64, 2 x v_xor_b32) beat a hand-written 9-instruction 32-bit form.
+    // A single wave issues one VALU instruction per ~4.8 cycles whether or not it depends on the previous one
+    // (measured), so a step costs its instruction count; chain_step() is 6.
     uint64_t h = seed;
     int64_t key_pos = 0;
     if (r < R) {
