@@ -1,0 +1,163 @@
+// kvcm_hip.hpp -- header-only C++ convenience layer over the C-ABI of libkvcm_hip.so, for host code that holds its
+// data in std::vector the way the reference's manager and client do. Function names and argument meaning follow the
+// reference interfaces cited below (paths relative to the reference root).
+//
+// Unlike the C-ABI underneath, these helpers allocate device memory, copy and WAIT for the stream: they are for
+// call sites that want a value back (a server thread answering one RPC, a trace converter, a test), not for the
+// asynchronous data path, which calls kvcm_hip_* directly on device buffers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdlib>
+#include <vector>
+
+#include "kvcm_hip.h"
+
+namespace kvcm {
+
+using TokenIdsVector = std::vector<int64_t>;  // kv_cache_manager/manager/cache_manager.h:55-56
+using KeyVector = std::vector<int64_t>;
+
+namespace detail {
+// Device buffer that frees itself; empty when the allocation failed.
+template <typename T>
+struct DeviceArray {
+    T *ptr = nullptr;
+    explicit DeviceArray(size_t n) {
+        if (n > 0 && hipMalloc(reinterpret_cast<void **>(&ptr), n * sizeof(T)) != hipSuccess) {
+            ptr = nullptr;
+        }
+    }
+    ~DeviceArray() {
+        if (ptr) {
+            (void)hipFree(ptr);
+        }
+    }
+    DeviceArray(const DeviceArray &) = delete;
+    DeviceArray &operator=(const DeviceArray &) = delete;
+};
+}  // namespace detail
+
+// GenKeyVector for a batch of requests in one launch: (*keys)[r] == GenKeyVector(requests[r], block_size) of
+// kv_cache_manager/manager/cache_manager.cc:76-87. Returns KVCM_OK, a KVCM_ERR_* code or a hipError_t.
+inline int32_t GenKeyVectors(const std::vector<TokenIdsVector> &requests, int64_t block_size,
+                             std::vector<KeyVector> *keys, hipStream_t stream = nullptr) {
+    if (!keys || block_size <= 0 || block_size > INT32_MAX || requests.size() > static_cast<size_t>(INT32_MAX)) {
+        return KVCM_ERR_INVALID_ARG;
+    }
+    const int32_t R = static_cast<int32_t>(requests.size());
+    keys->assign(requests.size(), KeyVector());
+    std::vector<int64_t> token_offsets(R + 1, 0), key_offsets(R + 1, 0);
+    for (int32_t r = 0; r < R; ++r) {
+        token_offsets[r + 1] = token_offsets[r] + static_cast<int64_t>(requests[r].size());
+        key_offsets[r + 1] = key_offsets[r] + static_cast<int64_t>(requests[r].size()) / block_size;
+    }
+    const int64_t n_tokens = token_offsets[R], n_keys = key_offsets[R];
+    if (n_keys == 0) {
+        return KVCM_OK;
+    }
+    std::vector<int64_t> flat(static_cast<size_t>(n_tokens));
+    for (int32_t r = 0; r < R; ++r) {
+        std::copy(requests[r].begin(), requests[r].end(), flat.begin() + token_offsets[r]);
+    }
+    detail::DeviceArray<int64_t> d_tokens(flat.size()), d_toff(token_offsets.size()), d_koff(key_offsets.size()),
+        d_keys(static_cast<size_t>(n_keys));
+    if (!d_tokens.ptr || !d_toff.ptr || !d_koff.ptr || !d_keys.ptr) {
+        return static_cast<int32_t>(hipErrorOutOfMemory);
+    }
+    hipError_t e = hipMemcpyAsync(d_tokens.ptr, flat.data(), flat.size() * 8, hipMemcpyHostToDevice, stream);
+    if (e == hipSuccess) {
+        e = hipMemcpyAsync(d_toff.ptr, token_offsets.data(), token_offsets.size() * 8, hipMemcpyHostToDevice, stream);
+    }
+    if (e == hipSuccess) {
+        e = hipMemcpyAsync(d_koff.ptr, key_offsets.data(), key_offsets.size() * 8, hipMemcpyHostToDevice, stream);
+    }
+    if (e != hipSuccess) {
+        return static_cast<int32_t>(e);
+    }
+    const int32_t rc = kvcm_hip_hash_tokens(d_tokens.ptr, d_toff.ptr, R, static_cast<int32_t>(block_size), 0,
+                                            d_keys.ptr, d_koff.ptr, stream);
+    if (rc != KVCM_OK) {
+        (void)hipStreamSynchronize(stream);
+        return rc;
+    }
+    std::vector<int64_t> flat_keys(static_cast<size_t>(n_keys));
+    e = hipMemcpyAsync(flat_keys.data(), d_keys.ptr, flat_keys.size() * 8, hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) {
+        e = hipStreamSynchronize(stream);
+    }
+    if (e != hipSuccess) {
+        return static_cast<int32_t>(e);
+    }
+    for (int32_t r = 0; r < R; ++r) {
+        (*keys)[r].assign(flat_keys.begin() + key_offsets[r], flat_keys.begin() + key_offsets[r + 1]);
+    }
+    return KVCM_OK;
+}
+
+// One request, the reference's own signature; an empty vector on error or when tokens is shorter than a block.
+inline KeyVector GenKeyVector(const TokenIdsVector &tokens, int64_t block_size) {
+    std::vector<KeyVector> out;
+    if (GenKeyVectors({tokens}, block_size, &out) != KVCM_OK || out.empty()) {
+        return {};
+    }
+    return out[0];
+}
+
+// kv_cache_manager/optimizer/trace_converter/trace_util.cc:47-56: one key per element, every key chained on the
+// one before.
+inline std::vector<int64_t> ApplyPrefixHash(const std::vector<int64_t> &hash_ids) {
+    return GenKeyVector(hash_ids, 1);
+}
+
+// SdkBufferCheckUtil::GetIovsCrc (kv_cache_manager/client/src/internal/sdk/sdk_buffer_check_util.cu:50-69):
+// cal_byte_size = min(min_cal_byte_size, iovs[0].size / 2); empty result when that is 0 or on error.
+inline std::vector<uint32_t> GetIovsCrc(const std::vector<kvcm_iov_device> &iovs_h, size_t min_cal_byte_size = 4,
+                                        hipStream_t stream = nullptr) {
+    if (iovs_h.empty()) {
+        return {};
+    }
+    const size_t cal = std::min(min_cal_byte_size, iovs_h.front().size / 2);
+    if (cal == 0) {
+        return {};
+    }
+    detail::DeviceArray<kvcm_iov_device> d_iovs(iovs_h.size());
+    detail::DeviceArray<uint32_t> d_crc(iovs_h.size());
+    if (!d_iovs.ptr || !d_crc.ptr) {
+        return {};
+    }
+    if (hipMemcpyAsync(d_iovs.ptr, iovs_h.data(), iovs_h.size() * sizeof(kvcm_iov_device), hipMemcpyHostToDevice,
+                       stream) != hipSuccess) {
+        return {};
+    }
+    if (kvcm_hip_iov_crc32(d_iovs.ptr, static_cast<int32_t>(iovs_h.size()), d_crc.ptr, cal, stream) != KVCM_OK) {
+        (void)hipStreamSynchronize(stream);
+        return {};
+    }
+    std::vector<uint32_t> crcs(iovs_h.size());
+    if (hipMemcpyAsync(crcs.data(), d_crc.ptr, crcs.size() * 4, hipMemcpyDeviceToHost, stream) != hipSuccess ||
+        hipStreamSynchronize(stream) != hipSuccess) {
+        return {};
+    }
+    return crcs;
+}
+
+// SdkBufferCheckUtil::GetBlocksHash (sdk_buffer_check_util.cc:11-28): one hash per block of iovs_per_block iovs.
+inline std::vector<int64_t> GetBlocksHash(const std::vector<kvcm_iov_device> &iovs_h, int32_t iovs_per_block,
+                                          size_t min_cal_byte_size = 4, hipStream_t stream = nullptr) {
+    const std::vector<uint32_t> crcs = GetIovsCrc(iovs_h, min_cal_byte_size, stream);
+    if (crcs.empty() || iovs_per_block <= 0) {
+        return {};
+    }
+    std::vector<int64_t> out(crcs.size() / iovs_per_block);
+    if (kvcm_blocks_hash_from_crcs(crcs.data(), static_cast<int64_t>(crcs.size()), iovs_per_block, out.data()) !=
+        KVCM_OK) {
+        return {};
+    }
+    return out;
+}
+
+}  // namespace kvcm

@@ -1,0 +1,188 @@
+// C++ tests of the C-ABI and of include/kvcm_hip.hpp on the GPU, checked against the C oracle (the checker is
+// linked here and only here). The CRC cases are the reference's own known answers
+// (kv_cache_manager/client/src/internal/sdk/test/sdk_buffer_check_util_test.cc:13-74) run through this library.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "kvcm_hip.hpp"
+#include "kvcm_oracle.h"
+
+static int g_failed = 0, g_run = 0;
+#define EXPECT(cond)                                                        \
+    do {                                                                    \
+        ++g_run;                                                            \
+        if (!(cond)) {                                                      \
+            ++g_failed;                                                     \
+            std::printf("FAILED %s:%d  %s\n", __FILE__, __LINE__, #cond);   \
+        }                                                                   \
+    } while (0)
+
+static std::vector<uint32_t> crc_of(const std::string &s, size_t min_cal) {
+    char *buffer = nullptr;
+    if (hipMalloc(reinterpret_cast<void **>(&buffer), s.size()) != hipSuccess) {
+        return {0xBAD};
+    }
+    (void)hipMemcpy(buffer, s.data(), s.size(), hipMemcpyHostToDevice);
+    std::vector<kvcm_iov_device> iovs_h{{buffer, s.size()}};
+    auto crcs = kvcm::GetIovsCrc(iovs_h, min_cal);
+    (void)hipFree(buffer);
+    return crcs;
+}
+
+static void test_crc_known_answers() {
+    EXPECT(crc_of("1234xxxxxxxx5678", 8) == std::vector<uint32_t>({0xDE28307C}));
+    EXPECT(crc_of("1234xxxxxxxx5678", 4) == std::vector<uint32_t>({0x9AE0DAAF}));
+    EXPECT(crc_of("1278", 4) == std::vector<uint32_t>({0xF639698C}));
+    EXPECT(crc_of("1", 4).empty());
+}
+
+static void test_blocks_hash() {
+    const size_t byte_size = 4 * 1024;
+    char *buffer = nullptr;
+    EXPECT(hipMalloc(reinterpret_cast<void **>(&buffer), byte_size) == hipSuccess);
+    std::string s(byte_size, 'a');
+    for (size_t i = 0; i < byte_size; ++i) {
+        s[i] = static_cast<char>('a' + i % 23);
+    }
+    (void)hipMemcpy(buffer, s.data(), byte_size, hipMemcpyHostToDevice);
+    std::vector<kvcm_iov_device> iovs;
+    std::vector<kvcm_ref_iov> ref_iovs;
+    for (int i = 0; i < 4; ++i) {
+        iovs.push_back({buffer + 1024 * i, 1024});
+        ref_iovs.push_back({s.data() + 1024 * i, 1024});
+    }
+    auto hashes = kvcm::GetBlocksHash(iovs, 2);
+    uint32_t crcs[4];
+    int64_t want[2];
+    kvcm_ref_iov_crc32(ref_iovs.data(), 4, crcs, 4);
+    kvcm_ref_blocks_hash_from_crcs(crcs, 4, 2, want);
+    EXPECT(hashes.size() == 2 && hashes[0] == want[0] && hashes[1] == want[1]);
+    (void)hipFree(buffer);
+}
+
+static void test_gen_key_vector() {
+    // known answer: tokens 0..63, block size 16, as the reference header computes them
+    kvcm::TokenIdsVector ramp(64);
+    for (int i = 0; i < 64; ++i) {
+        ramp[i] = i;
+    }
+    auto keys = kvcm::GenKeyVector(ramp, 16);
+    EXPECT(keys == kvcm::KeyVector({6556265598806870907LL, 1204744731699469120LL, -7610010845176483469LL,
+                                    2681637840371060507LL}));
+    EXPECT(kvcm::GenKeyVector({1, 2, 3}, 4).empty());
+    EXPECT(kvcm::GenKeyVector({}, 16).empty());
+    EXPECT(kvcm::GenKeyVector({456}, 1) == kvcm::KeyVector({-7046029254386352675LL}));
+
+    std::mt19937_64 rng(7);
+    std::vector<kvcm::TokenIdsVector> reqs;
+    for (int r = 0; r < 150; ++r) {
+        kvcm::TokenIdsVector t(rng() % 700);
+        for (auto &v : t) {
+            v = static_cast<int64_t>(rng());
+        }
+        reqs.push_back(t);
+    }
+    for (int64_t bs : {16, 7, 64}) {
+        std::vector<kvcm::KeyVector> got;
+        EXPECT(kvcm::GenKeyVectors(reqs, bs, &got) == KVCM_OK);
+        bool same = got.size() == reqs.size();
+        for (size_t r = 0; same && r < reqs.size(); ++r) {
+            kvcm::KeyVector want(reqs[r].size() / bs);
+            kvcm_ref_gen_key_vector(reqs[r].data(), static_cast<int64_t>(reqs[r].size()), bs, 0, want.data());
+            same = got[r] == want;
+        }
+        EXPECT(same);
+    }
+    // ApplyPrefixHash == the chain with one element per key
+    kvcm::TokenIdsVector ids(reqs[3].begin(), reqs[3].end());
+    std::vector<int64_t> want(ids.size()), off{0, static_cast<int64_t>(ids.size())};
+    kvcm_ref_prefix_chain(ids.data(), off.data(), 1, want.data());
+    EXPECT(kvcm::ApplyPrefixHash(ids) == want);
+    std::vector<kvcm::KeyVector> none;
+    EXPECT(kvcm::GenKeyVectors(reqs, 0, &none) == KVCM_ERR_INVALID_ARG);
+}
+
+static void test_gather_scatter_c_abi() {
+    // 3 layers x K/V, T = 16, rows of 256 bytes, 40 pool blocks, 9 work blocks in scrambled staging slots
+    const int P = 6, T = 16, B = 9, slots = 12, nblk = 40;
+    const int64_t row = 256, tile = T * row, blk = P * tile;
+    std::mt19937 rng(5);
+    std::vector<std::vector<uint8_t>> pools(P, std::vector<uint8_t>(nblk * tile));
+    for (auto &p : pools) {
+        for (auto &b : p) {
+            b = static_cast<uint8_t>(rng());
+        }
+    }
+    std::vector<int32_t> idx(B * T), sidx(B);
+    for (int b = 0; b < B; ++b) {
+        sidx[b] = (b * 5 + 3) % slots;
+        for (int t = 0; t < T; ++t) {
+            idx[b * T + t] = static_cast<int32_t>(rng() % (nblk * T));
+        }
+    }
+    std::vector<uint8_t> want(slots * blk, 0x6B), got(slots * blk, 0x6B);
+    std::vector<const void *> table_h(P);
+    for (int p = 0; p < P; ++p) {
+        table_h[p] = pools[p].data();
+    }
+    EXPECT(kvcm_ref_batch_gather(table_h.data(), P, want.data(), blk, idx.data(), sidx.data(), B, T, row) == 0);
+
+    std::vector<void *> d_pools(P);
+    for (int p = 0; p < P; ++p) {
+        EXPECT(hipMalloc(&d_pools[p], pools[p].size()) == hipSuccess);
+        (void)hipMemcpy(d_pools[p], pools[p].data(), pools[p].size(), hipMemcpyHostToDevice);
+    }
+    void **d_table;
+    int32_t *d_idx, *d_sidx;
+    uint8_t *d_stage;
+    EXPECT(hipMalloc(reinterpret_cast<void **>(&d_table), P * sizeof(void *)) == hipSuccess);
+    EXPECT(hipMalloc(reinterpret_cast<void **>(&d_idx), idx.size() * 4) == hipSuccess);
+    EXPECT(hipMalloc(reinterpret_cast<void **>(&d_sidx), sidx.size() * 4) == hipSuccess);
+    EXPECT(hipMalloc(reinterpret_cast<void **>(&d_stage), got.size()) == hipSuccess);
+    (void)hipMemcpy(d_table, d_pools.data(), P * sizeof(void *), hipMemcpyHostToDevice);
+    (void)hipMemcpy(d_idx, idx.data(), idx.size() * 4, hipMemcpyHostToDevice);
+    (void)hipMemcpy(d_sidx, sidx.data(), sidx.size() * 4, hipMemcpyHostToDevice);
+    (void)hipMemcpy(d_stage, got.data(), got.size(), hipMemcpyHostToDevice);
+    hipStream_t stream;
+    EXPECT(hipStreamCreate(&stream) == hipSuccess);
+    EXPECT(kvcm_hip_batch_gather(d_table, P, d_stage, blk, d_idx, d_sidx, B, T, row, 0, stream) == KVCM_OK);
+    EXPECT(hipStreamSynchronize(stream) == hipSuccess);
+    (void)hipMemcpy(got.data(), d_stage, got.size(), hipMemcpyDeviceToHost);
+    EXPECT(got == want);
+    // a capped grid (the reference's sm_count = 3) gives the same bytes
+    (void)hipMemset(d_stage, 0x6B, got.size());
+    EXPECT(kvcm_hip_batch_gather(d_table, P, d_stage, blk, d_idx, d_sidx, B, T, row, 3, stream) == KVCM_OK);
+    EXPECT(hipStreamSynchronize(stream) == hipSuccess);
+    (void)hipMemcpy(got.data(), d_stage, got.size(), hipMemcpyDeviceToHost);
+    EXPECT(got == want);
+    EXPECT(kvcm_hip_batch_gather(d_table, P, d_stage, blk - 1, d_idx, d_sidx, B, T, row, 0, stream) ==
+           KVCM_ERR_INVALID_ARG);
+    EXPECT(std::string(kvcm_hip_error_string(KVCM_ERR_TOO_LARGE)).size() > 0);
+    for (auto p : d_pools) {
+        (void)hipFree(p);
+    }
+    (void)hipFree(d_table);
+    (void)hipFree(d_idx);
+    (void)hipFree(d_sidx);
+    (void)hipFree(d_stage);
+    (void)hipStreamDestroy(stream);
+}
+
+int main() {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
+        std::printf("no GPU\n");
+        return 2;
+    }
+    test_crc_known_answers();
+    test_blocks_hash();
+    test_gen_key_vector();
+    test_gather_scatter_c_abi();
+    std::printf("%d checks, %d failed\n", g_run, g_failed);
+    return g_failed == 0 ? 0 : 1;
+}

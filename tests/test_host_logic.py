@@ -125,3 +125,58 @@ def test_signatures_match_the_reference_operators():
                                                                           "src_tensor", "token_indices"]
     assert list(inspect.signature(CopyBufferAllocator.__init__).parameters) == ["self", "device", "dtype", "shape",
                                                                                 "max_count"]
+
+
+def _vllm_caches(L=3, nblk=8, T=16, H=2, hd=64, dtype=torch.float16):
+    return {f"model.layers.{l}.attn": torch.zeros(2, nblk, T, H, hd, dtype=dtype) for l in range(L)}
+
+
+def test_register_kv_caches_pointer_order_and_spec_size():
+    # v1_connector.py:360-445: layer-major, K before V; slot shape [layers, 2, manager_block, heads*dim]
+    from tair_kvcache_amd import connector
+    kv = _vllm_caches()
+    info = connector.register_kv_caches(kv, manager_block_size=64, local_block_size=16, tp_rank=1, tp_size=2)
+    want = []
+    for t in kv.values():
+        want += [t[0].data_ptr(), t[1].data_ptr()]
+    assert info.all_kvcache_ptr_tensor_gpu.tolist() == want
+    assert info.kvcache_ptr_tensor_cpu.tolist() == [t.data_ptr() for t in kv.values()]
+    assert info.per_manager_location_spec_shape == (3, 2, 64, 128)
+    assert info.per_manager_location_spec_byte_size == 3 * 2 * 64 * 128 * 2
+    assert info.per_token_per_layer_dim_size == 128 and info.local_token_num == 8 * 16
+    assert (info.layer_num, info.tp_rank, info.tp_size, info.dtype) == (3, 1, 2, torch.float16)
+    # V of a layer sits block_num * block_size rows after K: the legacy [2, total, H] view of the same tensor
+    assert want[1] - want[0] == 8 * 16 * 128 * 2
+
+
+def test_register_kv_caches_mla_one_pointer_per_layer():
+    from tair_kvcache_amd import connector
+    kv = {f"l{l}": torch.zeros(32, 128, 576, dtype=torch.uint8) for l in range(4)}
+    info = connector.register_kv_caches(kv, manager_block_size=128, local_block_size=128, use_mla=True)
+    assert info.all_kvcache_ptr_tensor_gpu.tolist() == [t.data_ptr() for t in kv.values()]
+    assert info.per_manager_location_spec_shape == (4, 1, 128, 576)
+    assert info.per_manager_location_spec_byte_size == 4 * 128 * 576
+    assert info.local_token_num == 32 * 128
+
+
+def test_register_kv_caches_rejects_what_the_reference_asserts_on():
+    from tair_kvcache_amd import connector
+    kv = _vllm_caches()
+    with pytest.raises(AssertionError):  # engine block size mismatch (v1_connector.py:365)
+        connector.register_kv_caches(kv, 16, 32)
+    bad = dict(kv)
+    bad["x"] = torch.zeros(2, 8, 16, 2, 128, dtype=torch.float16)[..., :64]  # not contiguous (:367)
+    with pytest.raises(AssertionError):
+        connector.register_kv_caches(bad, 16, 16)
+    with pytest.raises(ValueError):
+        connector.register_kv_caches({}, 16, 16)
+
+
+def test_generate_blocks_idx_bounds_check_runs_on_the_host():
+    # the reference asserts per token (v1_connector.py:315); here the same condition is checked before any launch
+    from tair_kvcache_amd import connector
+    with pytest.raises(AssertionError):
+        connector.generate_blocks_idx([4], [0, 1, 2, 3], 64, 16, device="cpu")  # tokens 256..319 need block 16
+    with pytest.raises(AssertionError):
+        connector.generate_blocks_idx([-1], [0, 1, 2, 3], 16, 16, device="cpu")
+    assert connector.generate_blocks_idx([], [0], 16, 16, device="cpu").shape == (0, 16)
