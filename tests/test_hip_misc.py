@@ -142,3 +142,106 @@ def test_save_then_load_through_the_transfer_manager(oracle):
     assert all(not v.view(torch.int16).any() for v in kv3.values())
     for m in (mgr, mgr2, mgr3):
         m.shutdown()
+
+
+def test_entry_points_can_be_captured_in_a_hip_graph(oracle):
+    """The C-ABI neither allocates nor synchronises, so a transfer task (hash + gather + scatter on device-resident
+    indices) can be captured once and replayed; every replay is checked against the eager result on fresh data, with
+    eager work and synchronisations between replays."""
+    from tair_kvcache_amd import hashing
+    from tair_kvcache_amd.kernel import batch_gather_scatter_helper as bgs
+    P, T, D, nblk, B = 16, 16, 256, 256, 64
+    rng = np.random.default_rng(1)
+    pool = torch.zeros((P, nblk * T, D), dtype=torch.int16, device="cuda")
+    pool2 = torch.zeros_like(pool)
+    table, table2 = ptr_table([pool[p] for p in range(P)]), ptr_table([pool2[p] for p in range(P)])
+    blocks = cases.block_table(nblk, B)
+    runs = dev((blocks * T).astype(np.int32))
+    slots = torch.arange(B, dtype=torch.int32, device="cuda")
+    staging = torch.zeros((B, P, T, D), dtype=torch.int16, device="cuda")
+    tokens = torch.zeros((8, 256), dtype=torch.int64, device="cuda")
+    toff = torch.arange(9, dtype=torch.int64, device="cuda") * 256
+    koff = torch.arange(9, dtype=torch.int64, device="cuda") * 16
+    keys = torch.zeros(8 * 16, dtype=torch.int64, device="cuda")
+
+    def task():
+        hashing.hash_tokens(tokens, 16, token_offsets=toff, keys=keys, key_offsets=koff)
+        bgs.paged_gather_kv_caches(table, staging, runs, slots, T, D, T)
+        bgs.paged_scatter_kv_caches(table2, staging, runs, slots, T, D, T)
+
+    task()  # warm-up outside the capture
+    sync()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        task()
+    for it in range(4):
+        new_pool = rng.integers(0, 65536, size=(P, nblk * T, D), dtype=np.uint16)
+        new_tok = rng.integers(0, 128256, size=(8, 256), dtype=np.int64)
+        pool.copy_(dev(new_pool))
+        tokens.copy_(dev(new_tok))
+        pool2.zero_()
+        staging.zero_()
+        keys.zero_()
+        sync()
+        graph.replay()
+        sync()
+        want = np.zeros((B, P, T, D), dtype=np.uint16)
+        tidx = cases.token_idx_from_blocks(blocks, T)
+        oracle.batch_gather([new_pool[p] for p in range(P)], want, tidx, None, T, D * 2)
+        assert (host(staging, np.uint16) == want).all(), it
+        touched = tidx.reshape(-1)
+        got2 = host(pool2, np.uint16)
+        assert (got2[:, touched] == new_pool[:, touched]).all(), it
+        wkeys, _ = oracle.hash_tokens(new_tok, 16)
+        assert (host(keys, np.int64) == wkeys).all(), it
+
+
+def test_concurrent_callers_on_their_own_streams(oracle):
+    """Sixteen host threads, each with its own stream, staging slots and index set, call gather, scatter and the hash at
+    once (the reference drives its kernels from a 32-thread pool, data_transfer.py:80-93). The library keeps no
+    mutable state, so every thread must get exactly its own answer."""
+    from concurrent.futures import ThreadPoolExecutor
+    from tair_kvcache_amd import hashing
+    from tair_kvcache_amd.kernel import batch_gather_scatter_helper as bgs
+    P, T, D, nblk, n_threads, per = 8, 16, 128, 512, 16, 24
+    pools = cases.pool_u16(P, nblk * T, D)
+    d_pools = [dev(p) for p in pools]
+    table = ptr_table(d_pools)
+    perm = cases.block_table(nblk, n_threads * per)
+    staging = torch.zeros((n_threads * per, P, T, D), dtype=torch.int16, device="cuda")
+    fresh = [torch.zeros_like(t) for t in d_pools]
+    table2 = ptr_table(fresh)
+    toks = cases.tokens(n_threads * 4, 512, 32000, seed=9)
+    d_toks = dev(toks)
+    keys_out = [None] * n_threads
+    sync()
+
+    def worker(i):
+        torch.cuda.set_device(0)
+        stream = torch.cuda.Stream()
+        blocks = perm[i * per:(i + 1) * per]
+        slots = list(range(i * per, (i + 1) * per))
+        tidx = cases.token_idx_from_blocks(blocks, T).reshape(-1).tolist()
+        with torch.cuda.stream(stream):
+            for _ in range(5):
+                bgs.batch_gather_kv_caches(table, staging, tidx, slots, T, D)
+                bgs.batch_scatter_kv_caches(table2, staging, tidx, slots, T, D)
+                keys_out[i], _ = hashing.hash_tokens(d_toks[i * 4:(i + 1) * 4], 16)
+        stream.synchronize()
+        return i
+
+    with ThreadPoolExecutor(max_workers=n_threads) as ex:
+        assert sorted(ex.map(worker, range(n_threads))) == list(range(n_threads))
+    sync()
+    tidx_all = cases.token_idx_from_blocks(perm, T)
+    want = np.zeros((n_threads * per, P, T, D), dtype=np.uint16)
+    oracle.batch_gather(pools, want, tidx_all, None, T, D * 2)
+    assert (host(staging, np.uint16) == want).all()
+    touched = np.zeros(nblk * T, dtype=bool)
+    touched[tidx_all.reshape(-1)] = True
+    for p in range(P):
+        g = host(fresh[p], np.uint16)
+        assert (g[touched] == pools[p][touched]).all() and not g[~touched].any()
+    wkeys, _ = oracle.hash_tokens(toks, 16)
+    for i in range(n_threads):
+        assert (host(keys_out[i], np.int64) == wkeys[i * 128:(i + 1) * 128]).all()
