@@ -306,3 +306,29 @@ def test_shape_errors_raise_value_error():
         bgs.batch_gather_kv_caches(table, st, [0] * 32, [0, 1], 16, 7)  # staging is not whole blocks
     bgs.batch_gather_kv_caches(table, st, [], [], 16, 8)  # empty batch is a no-op
     sync()
+
+
+def test_block_major_pools_are_the_one_array_case(oracle):
+    """Engines whose pool is already block-major -- TRT-LLM's [blocks, layers, K|V, heads*dim*tokens]
+    (trtllm/connector.py:173-179) or a page-first host pool -- need no transposition: the pool is ONE array whose
+    'rows' are whole blocks, so the same entry point moves them with P = 1, T = 1 and block ids as slots."""
+    bgs = _ops()
+    nblk, layers, kvf, block_elems, B = 96, 4, 2, 8 * 64 * 32, 40
+    rng = np.random.default_rng(1)
+    pool = rng.integers(0, 65536, size=(nblk, layers * kvf * block_elems), dtype=np.uint16)
+    ids = cases.block_table(nblk, B)
+    want = np.zeros((B, 1, 1, pool.shape[1]), dtype=np.uint16)
+    oracle.batch_gather([pool], want, ids, None, 1, pool.shape[1] * 2)
+    assert (want[:, 0, 0] == pool[ids]).all()
+    d_pool = dev(pool)
+    table = ptr_table([d_pool])
+    st = torch.zeros((B, 1, 1, pool.shape[1]), dtype=torch.int16, device="cuda")
+    bgs.batch_gather_kv_caches(table, st, ids.tolist(), list(range(B)), 1, pool.shape[1])
+    sync()
+    assert (host(st, np.uint16) == want).all()
+    fresh = torch.zeros_like(d_pool)
+    bgs.batch_scatter_kv_caches(ptr_table([fresh]), st, ids.tolist(), list(range(B)), 1, pool.shape[1])
+    sync()
+    g = host(fresh, np.uint16)
+    rest = np.setdiff1d(np.arange(nblk), ids)
+    assert (g[ids] == pool[ids]).all() and not g[rest].any()
