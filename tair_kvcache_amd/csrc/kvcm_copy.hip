@@ -193,6 +193,7 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
         if (RUN == kRunPerGroup) {
             slot_shared = runs_b[r_first];
         } else if (RUN == kRunPerWave) {
+            // one chunk per thread: a wave's 64 chunks start at a multiple of 64 and lie inside one run
             r_shared = __builtin_amdgcn_readfirstlane(fast_div(cc_first + (threadIdx.x & ~63u), a.div_run));
             slot_shared = runs_b[r_shared];
         }
@@ -399,7 +400,7 @@ int32_t launch_copy(const kvcm_copy_desc *d, bool scatter, hipStream_t stream) {
     const uint32_t g32 = static_cast<uint32_t>(grid);
     if (cs == 16 && uni_tile && a.chunks_per_run % kSpan == 0) {
         launch_span<16, true, kRunPerGroup>(a, d, scatter, g32, stream);
-    } else if (cs == 16 && uni_tile && a.chunks_per_run % 64 == 0) {
+    } else if (cs == 16 && uni_tile && kCPT == 1 && a.chunks_per_run % 64 == 0) {
         launch_span<16, true, kRunPerWave>(a, d, scatter, g32, stream);
     } else if (cs == 16 && uni_tile) {
         launch_span<16, true, kRunPerThread>(a, d, scatter, g32, stream);

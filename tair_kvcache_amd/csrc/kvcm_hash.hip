@@ -74,7 +74,7 @@ struct LoaderCtx {
 };
 
 // Loader, fast form: 16-byte BUFFER loads. One load instruction covers 64 / kLPR request rows with kLPR lanes
-// each, so a tile takes kNL loads per lane (16 for int64 tokens, 8 for int32). The buffer resource spans from the
+// each, so a tile takes kNL loads per lane (32 for int64 tokens, 16 for int32). The buffer resource spans from the
 // workgroup's first token to the end of the batch: the hardware returns zeros past the end instead of faulting, so
 // the loads need no clamp, and a load costs two instructions (offset add + buffer_load_dwordx4). Positions past a
 // request's own last hashed token read a neighbour's tokens; the chain wave never consumes those entries.
