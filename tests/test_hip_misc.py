@@ -45,15 +45,18 @@ def test_iov_crc_and_block_hash_match_oracle(oracle):
 class FakeTransferClient:
     """Keeps blocks in a dict keyed by URI; stands in for TransferClient (transfer_client.h:19-21)."""
 
-    def __init__(self, fail_load=False):
+    def __init__(self, fail_load=False, fail_save=False):
         self.store = {}
         self.fail_load = fail_load
+        self.fail_save = fail_save
         self.lock = threading.Lock()
 
     def SaveKvCaches(self, uris, buffers):
         from tair_kvcache_amd.client_types import ClientErrorCode
         if len(uris) != len(buffers) or not uris:
             return (ClientErrorCode.ER_INVALID_PARAMS, [])
+        if self.fail_save:
+            return (ClientErrorCode.ER_SDKWRITE_ERROR, [])
         import ctypes
         with self.lock:
             for uri, buf in zip(uris, buffers):
@@ -140,7 +143,15 @@ def test_save_then_load_through_the_transfer_manager(oracle):
     assert res3[0] == [[ClientErrorCode.ER_SDKREAD_ERROR] * 4] and alloc._inuse_count == 0
     sync()
     assert all(not v.view(torch.int16).any() for v in kv3.values())
-    for m in (mgr, mgr2, mgr3):
+    # a failed save reports the client's code for every block of the task and returns the slots
+    mgr4 = connector.DataTransferManager(info, T, alloc, FakeTransferClient(fail_save=True), max_workers=2)
+    done4 = threading.Event()
+    res4 = []
+    mgr4.submit_task(mgr4.save_task, connector.MultiResult(1, lambda r: (res4.append(r), done4.set())), 0, uris[:3],
+                     idx_h[:3].tolist(), None)
+    assert done4.wait(60)
+    assert res4[0] == [[ClientErrorCode.ER_SDKWRITE_ERROR] * 3] and alloc._inuse_count == 0
+    for m in (mgr, mgr2, mgr3, mgr4):
         m.shutdown()
 
 
@@ -245,3 +256,73 @@ def test_concurrent_callers_on_their_own_streams(oracle):
     wkeys, _ = oracle.hash_tokens(toks, 16)
     for i in range(n_threads):
         assert (host(keys_out[i], np.int64) == wkeys[i * 128:(i + 1) * 128]).all()
+
+
+class DeviceStagingClient:
+    """A transfer client for staging slots that live in HBM: iovs arrive as MemoryType.GPU and are resolved back to
+    slots of the allocator's backing tensor (a real SDK would hipMemcpyAsync from iov.base)."""
+
+    def __init__(self, alloc):
+        self.alloc = alloc
+        self.store = {}
+
+    def _slot(self, iov):
+        from tair_kvcache_amd.client_types import MemoryType
+        assert iov.type == MemoryType.GPU and iov.size == self.alloc.slot_nbytes
+        off = iov.base - self.alloc._raw_buffer.data_ptr()
+        assert off % self.alloc.slot_nbytes == 0
+        return off // self.alloc.slot_nbytes
+
+    def SaveKvCaches(self, uris, buffers):
+        from tair_kvcache_amd.client_types import ClientErrorCode
+        for uri, buf in zip(uris, buffers):
+            self.store[uri] = self.alloc._raw_buffer[self._slot(buf.iovs[0])].cpu().clone()
+        return (ClientErrorCode.ER_OK, list(uris))
+
+    def LoadKvCaches(self, uris, buffers):
+        from tair_kvcache_amd.client_types import ClientErrorCode
+        for uri, buf in zip(uris, buffers):
+            self.alloc._raw_buffer[self._slot(buf.iovs[0])].copy_(self.store[uri])
+        torch.cuda.synchronize()
+        return ClientErrorCode.ER_OK
+
+
+def test_transfer_manager_with_staging_in_hbm(oracle):
+    """The same save/load choreography with the staging pool on the GPU: slots are handed over as GPU iovs."""
+    from tair_kvcache_amd import connector
+    from tair_kvcache_amd.client_types import ClientErrorCode
+    from tair_kvcache_amd.kernel.gather_scatter_helper import CopyBufferAllocator
+    L, nblk, T_eng, T_mgr, H, hd = 3, 64, 16, 32, 4, 32
+    rng = np.random.default_rng(4)
+    np_caches = [rng.integers(0, 65536, size=(2, nblk, T_eng, H, hd), dtype=np.uint16) for _ in range(L)]
+    kv = {f"layer{l}": dev(np_caches[l]).view(torch.float16) for l in range(L)}
+    info = connector.register_kv_caches(kv, manager_block_size=T_mgr, local_block_size=T_eng)
+    alloc = CopyBufferAllocator(torch.device("cuda"), torch.float16, list(info.per_manager_location_spec_shape), 16)
+    client = DeviceStagingClient(alloc)
+    mgr = connector.DataTransferManager(info, T_mgr, alloc, client, max_workers=2)
+    local_block_ids = cases.block_table(nblk, 24).tolist()  # 24 engine blocks = 12 manager blocks of 32 tokens
+    idx = connector.generate_blocks_idx(list(range(12)), local_block_ids, T_mgr, T_eng)
+    uris = [f"mem://blk{i}" for i in range(12)]
+    done = threading.Event()
+    res = []
+    mgr.submit_task(mgr.save_task, connector.MultiResult(1, lambda r: (res.append(r), done.set())), 0, uris, idx, None)
+    assert done.wait(60) and res[0] == [[ClientErrorCode.ER_OK] * 12]
+    pools = [np_caches[l][k].reshape(nblk * T_eng, H * hd) for l in range(L) for k in (0, 1)]
+    want = np.zeros((12, 2 * L, T_mgr, H * hd), dtype=np.uint16)
+    oracle.batch_gather(pools, want, host(idx, np.int32), None, T_mgr, H * hd * 2)
+    for i, uri in enumerate(uris):
+        assert (client.store[uri].view(torch.int16).numpy().view(np.uint16).reshape(2 * L, T_mgr, H * hd) == want[i]).all()
+    kv2 = {k: torch.zeros_like(v) for k, v in kv.items()}
+    mgr2 = connector.DataTransferManager(connector.register_kv_caches(kv2, T_mgr, T_eng), T_mgr, alloc, client,
+                                         max_workers=2)
+    done2 = threading.Event()
+    res2 = []
+    mgr2.submit_task(mgr2.load_task, connector.MultiResult(1, lambda r: (res2.append(r), done2.set())), 0, uris, idx)
+    assert done2.wait(60) and res2[0] == [[ClientErrorCode.ER_OK] * 12]
+    touched = np.array(local_block_ids)
+    for l in range(L):
+        g = host(kv2[f"layer{l}"].view(torch.int16), np.uint16)
+        assert (g[:, touched] == np_caches[l][:, touched]).all()
+    assert alloc._inuse_count == 0
+    mgr.shutdown()
+    mgr2.shutdown()
