@@ -31,11 +31,14 @@ namespace {
 #define KVCM_HASH_TILE_TOKENS 64
 #endif
 
-constexpr int kLoaders = KVCM_HASH_LOADERS;   // loader waves
+// Loader waves. Three, so that the four waves of a workgroup sit on the four SIMDs of a CU: the chain wave needs about
+// 280 VGPRs (two register sets of 64 pre-added terms) and must not share its SIMD's register file. More loaders were
+// measured with 32-token tiles (where the registers fit): no gain at 16 384 requests, 5 % slower for one batch.
+constexpr int kLoaders = KVCM_HASH_LOADERS;
 constexpr int kThreads = 64 * (1 + kLoaders);
 constexpr int kReqs = 64;                     // requests per workgroup = lanes of the chain wave
 constexpr int kTT = KVCM_HASH_TILE_TOKENS;    // tokens per request per tile
-constexpr int kRing = kLoaders;               // LDS tiles in the ring: loader lw always fills slot lw
+constexpr int kRing = 3;                      // LDS tiles in the ring: computed on, prefetched from, written to
 constexpr int kPad = 2;                       // keeps rows 16-byte aligned (b128 reads) and spreads banks
 constexpr int kPerLane = kReqs * kTT / 64;  // tile elements per loader lane
 
@@ -155,14 +158,16 @@ struct GlobalLoader {
     }
 };
 
-// A loader wave's whole life. Loader lw owns tiles lw, lw + 3, ... and ring slot lw. Tiles 0 and 1 are published
-// before the first barrier: the chain wave computes on tile k while its LDS reads of tile k+1 are already in
-// flight, so tile k+2 is what gets written during iteration k. Loads are issued AFTER a barrier, while the chain
-// wave is busy, and stay in flight for about two tile periods.
+// A loader wave's whole life. Loader lw owns tiles lw, lw + kLoaders, ...; tile t lives in ring slot t % kRing.
+// Tiles 0 and 1 are published before the first barrier: the chain wave computes on tile k while its LDS reads of
+// tile k+1 are already in flight, so tile k+2 is what gets written during iteration k (its slot held tile k-1,
+// which the chain wave pulled into registers an iteration ago). A loader issues the loads of its next tile right
+// AFTER the barrier that published its previous one, so they stay in flight for kLoaders - 1 tile periods while the
+// data waits in the loader's registers, not in LDS: more loaders = more bytes in flight per CU at no LDS cost.
 template <typename Loader, typename TokT>
 __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t (*s_tile)[kReqs][kTT + kPad],
                                            int64_t lw, int64_t ntiles, uint32_t lane) {
-    static_assert(kRing == kLoaders, "loader lw always fills ring slot lw");
+    static_assert(kRing == 3 && kLoaders >= 3, "three ring slots: computed on, prefetched from, written to");
     Loader ld;
     ld.setup(ctx, lane);
     if (lw < ntiles) {
@@ -176,13 +181,15 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
         ld.issue((lw + kLoaders) * kTT);
     }
     int64_t turn = 2 % kLoaders;  // loader whose tile is due: (k + 2) % kLoaders
+    int slot = 2;                 // ring slot of that tile: (k + 2) % kRing
     for (int64_t k = 0; k < ntiles; ++k) {
         const int64_t nxt = k + 2;  // tile that must be in LDS when this iteration ends
         const bool mine = turn == lw && nxt < ntiles;
-        turn = turn + 1 == kLoaders ? 0 : turn + 1;
         if (mine) {
-            ld.store(s_tile[lw]);
+            ld.store(s_tile[slot]);
         }
+        turn = turn + 1 == kLoaders ? 0 : turn + 1;
+        slot = slot + 1 == kRing ? 0 : slot + 1;
         lds_barrier();
         if (mine && nxt + kLoaders < ntiles) {
             ld.issue((nxt + kLoaders) * kTT);
