@@ -314,6 +314,11 @@ static void copy_one_block(const kvcm_ref_copy_desc *d, int32_t b, int scatter) 
             if (d->slot_limit > 0 && s >= d->slot_limit) {
                 continue;
             }
+            if (s < 0) {
+                /* No reference counterpart (a negative index is out of bounds there): the library's contract
+                 * skips such runs, e.g. the -1 entries kvcm_hip_generate_blocks_idx writes past the block list. */
+                continue;
+            }
             uint8_t *row = pool + s * d->row_bytes;
             uint8_t *st = tile + (int64_t)r * run_bytes;
             if (scatter) {

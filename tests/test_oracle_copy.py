@@ -157,6 +157,16 @@ def test_legacy_layout_equals_batch_on_views(oracle):
                                entry_stride_bytes=total * H * 2, slot_limit=total)
     oracle.gather_ex(d)
     assert (dst3[:, :, [1, 7]] == 0x7777).all() and (dst3[:, :, 0] == np.stack([c[:, idx[0]] for c in caches])).all()
+    # negative rows (the -1 that generate_blocks_idx writes past the local blocks) are skipped too, limit or not
+    for limit in (total, 0):
+        idx_neg = idx.copy()
+        idx_neg[[0, 9]] = [-1, -7]
+        dst4 = np.full((L, 2, T, H), 0x3333, dtype=np.uint16)
+        d, keep = oracle.make_desc(caches, dst4, idx_neg, None, 1, T, H * 2, ptrs_per_entry=2,
+                                   entry_stride_bytes=total * H * 2, slot_limit=limit)
+        oracle.gather_ex(d)
+        assert (dst4[:, :, [0, 9]] == 0x3333).all()
+        assert (np.delete(dst4, [0, 9], axis=2) == np.delete(dst, [0, 9], axis=2)).all()
 
 
 def test_trailer_interleave_bruteforce(oracle):
