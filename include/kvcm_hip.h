@@ -197,6 +197,39 @@ int32_t kvcm_hip_generate_blocks_idx(const int32_t *d_manager_block_idxes, int32
                                      kvcm_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * Which blocks of a batch have to be saved
+ * ------------------------------------------------------------------------------------------------ */
+
+/*
+ * In-batch duplicate detection on block keys: d_first_idx[i] = the smallest j with d_keys[j] == d_keys[i]
+ * (so d_first_idx[i] == i marks the first occurrence); d_is_repeat (uint8 [n], may be NULL) gets 1 where a smaller
+ * index holds the same key, 0 otherwise -- the polarity of the manager's block mask, "true = nothing to save".
+ * No counterpart in the reference: there a block that several requests share is filtered by the manager, one
+ * StartWriteCache call per request against the metadata index (FilterWriteCache,
+ * kv_cache_manager/manager/cache_manager.cc:589-635); this is the batched, client-side form for connectors that
+ * compute block_keys themselves (kvcm_hip_hash_tokens) and save a whole batch of requests at once.
+ * d_workspace: device scratch of at least kvcm_hip_first_occurrence_workspace_bytes(n) bytes, 4-byte aligned,
+ * contents irrelevant before and undefined after. n <= 2^30. The result does not depend on scheduling.
+ */
+int64_t kvcm_hip_first_occurrence_workspace_bytes(int64_t n);
+int32_t kvcm_hip_first_occurrence(const int64_t *d_keys, int64_t n, void *d_workspace, int64_t workspace_bytes,
+                                  int32_t *d_first_idx, uint8_t *d_is_repeat, kvcm_stream_t stream);
+
+/*
+ * Indices of the blocks to save, ascending: every i < n with d_mask[i] == 0 (and d_mask2[i] == 0 when d_mask2 is
+ * not NULL) is appended to d_indices (int32, room for n entries); their number goes to *d_count (device int32).
+ * Replaces: TairKvCacheConnector.parse_block_mask_to_save_indices, bool_masks branch
+ *           kv_cache_manager/py_connector/vllm/v1_connector.py:835-850 ("False = has to be saved"); the offset
+ *           branch (:839-842) is the mask that is 1 below the offset.
+ * d_mask2 lets the caller combine the manager's mask with d_is_repeat of kvcm_hip_first_occurrence.
+ * d_workspace: at least kvcm_hip_mask_to_indices_workspace_bytes(n) bytes, 4-byte aligned. n <= 2^30.
+ */
+int64_t kvcm_hip_mask_to_indices_workspace_bytes(int64_t n);
+int32_t kvcm_hip_mask_to_indices(const uint8_t *d_mask, const uint8_t *d_mask2, int64_t n, void *d_workspace,
+                                 int64_t workspace_bytes, int32_t *d_indices, int32_t *d_count,
+                                 kvcm_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
  * Buffer check (debug aid of the transfer client)
  * ------------------------------------------------------------------------------------------------ */
 

@@ -508,3 +508,57 @@ int32_t kvcm_ref_blocks_hash_from_crcs(const uint32_t *crcs, int64_t n_crcs, int
     }
     return 0;
 }
+
+/* ------------------------------------------------------------------ which blocks to save */
+
+struct key_pos {
+    int64_t key;
+    int32_t pos;
+};
+
+static int key_pos_less(const void *a, const void *b) {
+    const struct key_pos *x = (const struct key_pos *)a, *y = (const struct key_pos *)b;
+    if (x->key != y->key) {
+        return x->key < y->key ? -1 : 1;
+    }
+    return x->pos < y->pos ? -1 : (x->pos > y->pos);
+}
+
+/* first_idx[i] = smallest j with keys[j] == keys[i]. No reference counterpart (the manager filters shared blocks
+ * request by request against its index, cache_manager.cc:589-635); stated by sorting (key, position) pairs. */
+int32_t kvcm_ref_first_occurrence(const int64_t *keys, int64_t n, int32_t *first_idx, uint8_t *is_repeat) {
+    if (n < 0 || (n > 0 && (!keys || !first_idx))) {
+        return -1;
+    }
+    struct key_pos *kp = (struct key_pos *)malloc(sizeof(struct key_pos) * (size_t)(n ? n : 1));
+    for (int64_t i = 0; i < n; i++) {
+        kp[i].key = keys[i];
+        kp[i].pos = (int32_t)i;
+    }
+    qsort(kp, (size_t)n, sizeof(struct key_pos), key_pos_less);
+    int32_t head = 0;
+    for (int64_t i = 0; i < n; i++) {
+        if (i == 0 || kp[i].key != kp[i - 1].key) {
+            head = kp[i].pos;
+        }
+        first_idx[kp[i].pos] = head;
+    }
+    free(kp);
+    for (int64_t i = 0; is_repeat && i < n; i++) {
+        is_repeat[i] = first_idx[i] != (int32_t)i;
+    }
+    return 0;
+}
+
+/* v1_connector.py:835-850, bool_masks branch: the indices whose mask entry is false, in order.
+ * mask2 (optional) is OR-ed in. Returns the number of indices written. */
+int64_t kvcm_ref_mask_to_indices(const uint8_t *mask, const uint8_t *mask2, int64_t n, int32_t *indices) {
+    int64_t count = 0;
+    for (int64_t idx = 0; idx < n; idx++) {
+        int is_saved = mask[idx] != 0 || (mask2 && mask2[idx] != 0);
+        if (!is_saved) {
+            indices[count++] = (int32_t)idx;
+        }
+    }
+    return count;
+}

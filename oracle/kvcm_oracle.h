@@ -106,6 +106,13 @@ int32_t kvcm_ref_iov_crc32(const kvcm_ref_iov *iovs, int32_t n, uint32_t *crc, s
 int32_t kvcm_ref_blocks_hash_from_crcs(const uint32_t *crcs, int64_t n_crcs, int32_t iovs_per_block,
                                        int64_t *out_hashes);
 
+/* In-batch first occurrence of every key (no reference counterpart; the manager's per-request filter is
+ * kv_cache_manager/manager/cache_manager.cc:589-635). is_repeat may be NULL. */
+int32_t kvcm_ref_first_occurrence(const int64_t *keys, int64_t n, int32_t *first_idx, uint8_t *is_repeat);
+
+/* parse_block_mask_to_save_indices, bool_masks branch: kv_cache_manager/py_connector/vllm/v1_connector.py:835-850. */
+int64_t kvcm_ref_mask_to_indices(const uint8_t *mask, const uint8_t *mask2, int64_t n, int32_t *indices);
+
 #ifdef __cplusplus
 }
 #endif

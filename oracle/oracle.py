@@ -12,6 +12,7 @@ Reference lines followed (paths relative to the reference root):
   legacy gather        kv_cache_manager/py_connector/kernel/gather_scatter_helper.py:10-107
   generate_blocks_idx  kv_cache_manager/py_connector/vllm/v1_connector.py:308-320
   iov CRC              kv_cache_manager/client/src/internal/sdk/sdk_buffer_check_util.cu:10-44
+  mask -> save indices kv_cache_manager/py_connector/vllm/v1_connector.py:835-850
 """
 import ctypes as C
 import os
@@ -105,6 +106,10 @@ def lib():
         L.kvcm_ref_iov_crc32.argtypes = [vp, i32, vp, C.c_size_t]
         L.kvcm_ref_blocks_hash_from_crcs.restype = i32
         L.kvcm_ref_blocks_hash_from_crcs.argtypes = [vp, i64, i32, vp]
+        L.kvcm_ref_first_occurrence.restype = i32
+        L.kvcm_ref_first_occurrence.argtypes = [vp, i64, vp, vp]
+        L.kvcm_ref_mask_to_indices.restype = i64
+        L.kvcm_ref_mask_to_indices.argtypes = [vp, vp, i64, vp]
         _lib = L
     return _lib
 
@@ -335,6 +340,41 @@ def py_generate_blocks_idx(manager_block_idxes, local_block_ids, T_mgr, T_eng):
             row.append(local_block_ids[tok // T_eng] * T_eng + tok % T_eng)
         out.append(row)
     return out
+
+
+# ---------------------------------------------------------------------------------------------- which blocks to save
+
+def first_occurrence(keys):
+    """first_idx[i] = smallest j with keys[j] == keys[i]; is_repeat[i] = first_idx[i] != i."""
+    k = np.ascontiguousarray(keys, dtype=np.int64)
+    first = np.zeros(len(k), dtype=np.int32)
+    rep = np.zeros(len(k), dtype=np.uint8)
+    rc = lib().kvcm_ref_first_occurrence(_p(k), len(k), _p(first), _p(rep))
+    assert rc == 0, rc
+    return first, rep
+
+
+def mask_to_indices(mask, mask2=None):
+    """Indices whose mask entries are all false (v1_connector.py:835-850, bool_masks branch)."""
+    a = np.ascontiguousarray(mask, dtype=np.uint8)
+    b = None if mask2 is None else np.ascontiguousarray(mask2, dtype=np.uint8)
+    out = np.zeros(len(a), dtype=np.int32)
+    n = lib().kvcm_ref_mask_to_indices(_p(a), _p(b), len(a), _p(out))
+    return out[:n]
+
+
+def py_parse_block_mask_to_save_indices(response, target_save_num):
+    """v1_connector.py:835-850 on the response dict, both branches."""
+    block_mask = response.get("block_mask", {})
+    save_indices = []
+    if "offset" in block_mask:
+        for idx in range(block_mask["offset"], target_save_num):
+            save_indices.append(idx)
+    else:
+        for idx, is_saved in enumerate(block_mask.get("bool_masks", {}).get("values", [])):
+            if not is_saved:
+                save_indices.append(idx)
+    return save_indices
 
 
 # ---------------------------------------------------------------------------------------------- buffer check

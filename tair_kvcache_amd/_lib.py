@@ -61,6 +61,10 @@ SIGNATURES = {
     "kvcm_hip_gather_ex": (i32, [C.POINTER(CopyDesc), vp]),
     "kvcm_hip_scatter_ex": (i32, [C.POINTER(CopyDesc), vp]),
     "kvcm_hip_generate_blocks_idx": (i32, [vp, i32, vp, i32, i32, i32, vp, vp, vp]),
+    "kvcm_hip_first_occurrence_workspace_bytes": (i64, [i64]),
+    "kvcm_hip_first_occurrence": (i32, [vp, i64, vp, i64, vp, vp, vp]),
+    "kvcm_hip_mask_to_indices_workspace_bytes": (i64, [i64]),
+    "kvcm_hip_mask_to_indices": (i32, [vp, vp, i64, vp, i64, vp, vp, vp]),
     "kvcm_hip_iov_crc32": (i32, [vp, i32, vp, sz, vp]),
     "kvcm_blocks_hash_from_crcs": (i32, [vp, i64, i32, vp]),
 }

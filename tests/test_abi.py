@@ -19,7 +19,9 @@ def test_header_declares_the_expected_entry_points():
     for must in ("kvcm_hip_hash_tokens", "kvcm_hip_hash_tokens_i32", "kvcm_hip_prefix_chain",
                  "kvcm_hip_sha256_first8_be", "kvcm_hip_batch_gather", "kvcm_hip_batch_scatter",
                  "kvcm_hip_paged_gather", "kvcm_hip_paged_scatter", "kvcm_hip_gather_ex", "kvcm_hip_scatter_ex",
-                 "kvcm_hip_generate_blocks_idx", "kvcm_hip_iov_crc32", "kvcm_blocks_hash_from_crcs"):
+                 "kvcm_hip_generate_blocks_idx", "kvcm_hip_iov_crc32", "kvcm_blocks_hash_from_crcs",
+                 "kvcm_hip_first_occurrence", "kvcm_hip_first_occurrence_workspace_bytes",
+                 "kvcm_hip_mask_to_indices", "kvcm_hip_mask_to_indices_workspace_bytes"):
         assert must in names
 
 
@@ -36,7 +38,8 @@ def test_every_prototype_cites_the_reference():
     text = open(os.path.join(ROOT, "include", "kvcm_hip.h")).read()
     for anchor in ("cache_manager.cc:76-87", "hash_util.h:8-24", "trace_util.cc:47-56", "connector.py:397-415",
                    "batch_gather_scatter_helper.py:33-136", "batch_gather_scatter_helper.py:139-248",
-                   "v1_connector.py:308-320", "sdk_buffer_check_util.cu:21-44", "sdk_buffer_check_util.cc:56-60"):
+                   "v1_connector.py:308-320", "sdk_buffer_check_util.cu:21-44", "sdk_buffer_check_util.cc:56-60",
+                   "v1_connector.py:835-850", "cache_manager.cc:589-635"):
         assert anchor in text, anchor
 
 
@@ -61,6 +64,14 @@ def test_argument_validation_needs_no_device():
     assert L.kvcm_hip_sha256_first8_be(None, None, 0, None, None) == _lib.OK
     assert L.kvcm_hip_iov_crc32(None, 1, None, 4, None) == _lib.ERR_INVALID_ARG
     assert L.kvcm_hip_generate_blocks_idx(p, 1, p, 1, 0, 16, p, None, None) == _lib.ERR_INVALID_ARG
+    assert L.kvcm_hip_first_occurrence_workspace_bytes(0) == 4096 and L.kvcm_hip_first_occurrence_workspace_bytes(513) == 2048 * 4
+    assert L.kvcm_hip_first_occurrence_workspace_bytes((1 << 30) + 1) == _lib.ERR_TOO_LARGE
+    assert L.kvcm_hip_first_occurrence(None, 0, None, 0, None, None, None) == _lib.OK
+    assert L.kvcm_hip_first_occurrence(None, 5, p, 1 << 20, p, None, None) == _lib.ERR_INVALID_ARG
+    assert L.kvcm_hip_first_occurrence(p, 5, p, 8, p, None, None) == _lib.ERR_INVALID_ARG  # workspace too small
+    assert L.kvcm_hip_mask_to_indices_workspace_bytes(1025) == 3 * 4
+    assert L.kvcm_hip_mask_to_indices(p, None, 5, p, 1 << 20, p, None, None) == _lib.ERR_INVALID_ARG  # no count
+    assert L.kvcm_hip_mask_to_indices(p, None, (1 << 30) + 1, p, 1 << 20, p, p, None) == _lib.ERR_TOO_LARGE
     assert _lib.error_string(_lib.ERR_INVALID_ARG) == "invalid argument"
     assert _lib.error_string(0) == "ok"
 
