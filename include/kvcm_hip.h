@@ -37,6 +37,7 @@ typedef void *kvcm_stream_t;
 #define KVCM_ERR_INVALID_ARG (-1) /* null pointer, non-positive size, inconsistent shape */
 #define KVCM_ERR_ALIGNMENT (-2)   /* an address or stride is not aligned as the entry point requires */
 #define KVCM_ERR_TOO_LARGE (-3)   /* a size exceeds what the launch geometry can express */
+#define KVCM_ERR_IO (-4)          /* a file could not be created, opened, grown, read or written */
 
 /* Library version: major*10000 + minor*100 + patch. */
 int32_t kvcm_hip_version(void);
@@ -256,6 +257,57 @@ int32_t kvcm_hip_iov_crc32(const kvcm_iov_device *d_iovs, int32_t n, uint32_t *d
  */
 int32_t kvcm_blocks_hash_from_crcs(const uint32_t *crcs, int64_t n_crcs, int32_t iovs_per_block,
                                    int64_t *out_hashes);
+
+/* ------------------------------------------------------------------------------------------------
+ * Staging slots <-> block files (host code; the step after gather and before scatter)
+ * ------------------------------------------------------------------------------------------------ */
+
+#define KVCM_MEMORY_CPU 0
+#define KVCM_MEMORY_GPU 1
+
+/* One contiguous piece of a block, in host or device memory.
+ * Mirrors: struct Iov  kv_cache_manager/client/include/common.h:102-110 (MemoryType :94-97). */
+typedef struct kvcm_iov {
+    uint8_t type;   /* KVCM_MEMORY_CPU or KVCM_MEMORY_GPU */
+    uint8_t ignore; /* non-zero: skip the bytes, still advance the file offset */
+    void *base;     /* NULL is skipped like an ignored iov */
+    size_t size;
+} kvcm_iov;
+
+typedef struct kvcm_file_store kvcm_file_store;
+
+/*
+ * Replaces: LocalFileSdk::Init  kv_cache_manager/client/src/internal/sdk/local_file_sdk.cc:68-85.
+ * byte_size_per_block must be positive. bounce_bytes = size of each pinned bounce buffer for device iovs (0 = 8 MiB);
+ * they, and a stream, are created on the first call that meets a device iov, per concurrent caller (at most 64), and
+ * live until the store is destroyed. sync_on_put != 0 ends every put with fdatasync, the counterpart of the
+ * reference's msync(MS_SYNC) (:362). A store may be used from many threads at once. This family of entry points does
+ * allocate and does block: it is file I/O.
+ */
+int32_t kvcm_file_store_create(int64_t byte_size_per_block, int64_t bounce_bytes, int32_t sync_on_put,
+                               kvcm_file_store **out);
+void kvcm_file_store_destroy(kvcm_file_store *store);
+
+/*
+ * Writes n_blocks blocks into ONE file: block b goes to byte offset blkids[b] * byte_size_per_block, its
+ * iov_counts[b] iovs (consecutive entries of `iovs`) back to back from there. The file and its parent directories
+ * are created when missing and the file is grown to (max blkid + 1) * byte_size_per_block, never shrunk.
+ * sizes[b] is the `size` parameter of the block's URI and must equal byte_size_per_block; an iov that would reach
+ * beyond the grown size is refused. Everything is checked before the first byte moves.
+ * Replaces: LocalFileSdk::Alloc + DoPut  local_file_sdk.cc:136-159,262-364 for one path group of Put (:115-133).
+ * Returns KVCM_OK, KVCM_ERR_INVALID_ARG (the reference's ER_INVALID_PARAMS cases), KVCM_ERR_IO
+ * (ER_FILE_IO_ERROR cases) or a positive hipError_t.
+ */
+int32_t kvcm_file_store_put(kvcm_file_store *store, const char *path, const uint64_t *blkids, const uint64_t *sizes,
+                            const int32_t *iov_counts, const kvcm_iov *iovs, int32_t n_blocks);
+
+/*
+ * Reads n_blocks blocks of ONE file into their iovs; the inverse of put. The file must exist; an iov that would reach
+ * beyond its end is refused (local_file_sdk.cc:221-224). Returns when the data are in place (device iovs included).
+ * Replaces: LocalFileSdk::DoGet  local_file_sdk.cc:161-260 for one path group of Get (:89-103).
+ */
+int32_t kvcm_file_store_get(kvcm_file_store *store, const char *path, const uint64_t *blkids, const uint64_t *sizes,
+                            const int32_t *iov_counts, const kvcm_iov *iovs, int32_t n_blocks);
 
 #ifdef __cplusplus
 }

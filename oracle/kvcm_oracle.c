@@ -24,11 +24,16 @@
  *         whose values name their own slot, scatter(gather) = identity, and canary guard bands.
  *   The trailer (per-block scale) interleave has no reference counterpart: brute force only.
  */
+#define _GNU_SOURCE
 #include "kvcm_oracle.h"
 
+#include <fcntl.h>
 #include <pthread.h>
 #include <stdlib.h>
 #include <string.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
 
 #define KVCM_GOLDEN 0x9e3779b97f4a7c15ULL
 
@@ -561,4 +566,111 @@ int64_t kvcm_ref_mask_to_indices(const uint8_t *mask, const uint8_t *mask2, int6
         }
     }
     return count;
+}
+
+/* ------------------------------------------------------------------ block files (host iovs only) */
+
+/* local_file_sdk.cc:262-364 (DoPut) after Alloc (:136-159): the file is created when missing, grown with fallocate
+ * to (max blkid + 1) * bsz, mapped, and every iov is memcpy'd to blkid * bsz + running offset; ignored or null
+ * iovs only advance the offset. Returns 0, -1 (the reference's invalid-parameter cases) or -4 (file I/O).
+ * The parent directory must exist (the tests make it). Like the reference, a failure half-way leaves the bytes
+ * already copied in the file. */
+int32_t kvcm_ref_file_put(const char *path, int64_t bsz, const uint64_t *blkids, const uint64_t *sizes,
+                          const int32_t *iov_counts, const kvcm_ref_fiov *iovs, int32_t n_blocks) {
+    if (n_blocks <= 0) {
+        return -1;
+    }
+    uint64_t max_blkid = 0, required_size = 0;
+    for (int32_t i = 0; i < n_blocks; i++) {
+        if ((uint64_t)bsz != sizes[i]) {
+            return -1;
+        }
+        if (blkids[i] > max_blkid) {
+            max_blkid = blkids[i];
+        }
+        if ((max_blkid + 1) * (uint64_t)bsz > required_size) {
+            required_size = (max_blkid + 1) * (uint64_t)bsz;
+        }
+    }
+    int fd = open(path, O_RDWR | O_CREAT, 0644);
+    if (fd < 0) {
+        return -4;
+    }
+    if (fallocate(fd, 0, 0, (off_t)required_size) != 0) {
+        close(fd);
+        return -4;
+    }
+    char *dst = (char *)mmap(NULL, required_size, PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+    if (dst == MAP_FAILED) {
+        close(fd);
+        return -4;
+    }
+    int32_t rc = 0;
+    int64_t first = 0;
+    for (int32_t i = 0; i < n_blocks && rc == 0; i++) {
+        uint64_t offset = blkids[i] * (uint64_t)bsz;
+        for (int32_t k = 0; k < iov_counts[i]; k++) {
+            const kvcm_ref_fiov *iov = &iovs[first + k];
+            if (offset + iov->size > required_size) {
+                rc = -1;
+                break;
+            }
+            if (!iov->ignore && iov->base && iov->size > 0) {
+                memcpy(dst + offset, iov->base, iov->size);
+            }
+            offset += iov->size;
+        }
+        first += iov_counts[i];
+    }
+    msync(dst, required_size, MS_SYNC);
+    munmap(dst, required_size);
+    close(fd);
+    return rc;
+}
+
+/* local_file_sdk.cc:161-260 (DoGet): the file must exist; iovs beyond its end are refused. */
+int32_t kvcm_ref_file_get(const char *path, int64_t bsz, const uint64_t *blkids, const uint64_t *sizes,
+                          const int32_t *iov_counts, const kvcm_ref_fiov *iovs, int32_t n_blocks) {
+    if (n_blocks <= 0) {
+        return -1;
+    }
+    int fd = open(path, O_RDONLY);
+    if (fd < 0) {
+        return -4;
+    }
+    struct stat st;
+    if (fstat(fd, &st) != 0) {
+        close(fd);
+        return -4;
+    }
+    size_t file_size = (size_t)st.st_size;
+    char *src = (char *)mmap(NULL, file_size, PROT_READ, MAP_PRIVATE, fd, 0);
+    if (src == MAP_FAILED) {
+        close(fd);
+        return -4;
+    }
+    int32_t rc = 0;
+    int64_t first = 0;
+    for (int32_t i = 0; i < n_blocks && rc == 0; i++) {
+        if ((uint64_t)bsz != sizes[i]) {
+            rc = -1;
+            break;
+        }
+        uint64_t offset = blkids[i] * (uint64_t)bsz;
+        for (int32_t k = 0; k < iov_counts[i]; k++) {
+            const kvcm_ref_fiov *iov = &iovs[first + k];
+            if (offset + iov->size > file_size) {
+                rc = -1;
+                break;
+            }
+            if (!iov->ignore && iov->base && iov->size > 0) {
+                memcpy(iov->base, src + offset, iov->size);
+            }
+            offset += iov->size;
+        }
+        first += iov_counts[i];
+    }
+    munmap(src, file_size);
+    close(fd);
+    return rc;
 }

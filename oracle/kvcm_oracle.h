@@ -113,6 +113,20 @@ int32_t kvcm_ref_first_occurrence(const int64_t *keys, int64_t n, int32_t *first
 /* parse_block_mask_to_save_indices, bool_masks branch: kv_cache_manager/py_connector/vllm/v1_connector.py:835-850. */
 int64_t kvcm_ref_mask_to_indices(const uint8_t *mask, const uint8_t *mask2, int64_t n, int32_t *indices);
 
+/* Iov (kv_cache_manager/client/include/common.h:102-110) for the block-file functions; host memory only here. */
+typedef struct kvcm_ref_fiov {
+    uint8_t type;
+    uint8_t ignore;
+    void *base;
+    size_t size;
+} kvcm_ref_fiov;
+
+/* LocalFileSdk::DoPut / DoGet on host iovs: kv_cache_manager/client/src/internal/sdk/local_file_sdk.cc:161-364. */
+int32_t kvcm_ref_file_put(const char *path, int64_t bsz, const uint64_t *blkids, const uint64_t *sizes,
+                          const int32_t *iov_counts, const kvcm_ref_fiov *iovs, int32_t n_blocks);
+int32_t kvcm_ref_file_get(const char *path, int64_t bsz, const uint64_t *blkids, const uint64_t *sizes,
+                          const int32_t *iov_counts, const kvcm_ref_fiov *iovs, int32_t n_blocks);
+
 #ifdef __cplusplus
 }
 #endif

@@ -13,6 +13,7 @@ Reference lines followed (paths relative to the reference root):
   generate_blocks_idx  kv_cache_manager/py_connector/vllm/v1_connector.py:308-320
   iov CRC              kv_cache_manager/client/src/internal/sdk/sdk_buffer_check_util.cu:10-44
   mask -> save indices kv_cache_manager/py_connector/vllm/v1_connector.py:835-850
+  block files          kv_cache_manager/client/src/internal/sdk/local_file_sdk.cc:161-364
 """
 import ctypes as C
 import os
@@ -106,6 +107,9 @@ def lib():
         L.kvcm_ref_iov_crc32.argtypes = [vp, i32, vp, C.c_size_t]
         L.kvcm_ref_blocks_hash_from_crcs.restype = i32
         L.kvcm_ref_blocks_hash_from_crcs.argtypes = [vp, i64, i32, vp]
+        for name in ("kvcm_ref_file_put", "kvcm_ref_file_get"):
+            getattr(L, name).restype = i32
+            getattr(L, name).argtypes = [C.c_char_p, i64, vp, vp, vp, vp, i32]
         L.kvcm_ref_first_occurrence.restype = i32
         L.kvcm_ref_first_occurrence.argtypes = [vp, i64, vp, vp]
         L.kvcm_ref_mask_to_indices.restype = i64
@@ -375,6 +379,42 @@ def py_parse_block_mask_to_save_indices(response, target_save_num):
             if not is_saved:
                 save_indices.append(idx)
     return save_indices
+
+
+# ---------------------------------------------------------------------------------------------- block files
+
+class FileIov(C.Structure):
+    """struct kvcm_ref_fiov."""
+    _fields_ = [("type", C.c_uint8), ("ignore", C.c_uint8), ("base", C.c_void_p), ("size", C.c_size_t)]
+
+
+def _file_call(fn, path, bsz, blocks, sizes=None):
+    """blocks: list of (blkid, [iov, ...]); an iov is a NumPy uint8 array (moved), an int n (n ignored bytes) or
+    ("null", n) (null base of n bytes). sizes: the URI `size` per block (default bsz)."""
+    n = len(blocks)
+    blkids = np.array([b[0] for b in blocks], dtype=np.uint64)
+    sz = np.array([bsz] * n if sizes is None else sizes, dtype=np.uint64)
+    counts = np.array([len(b[1]) for b in blocks], dtype=np.int32)
+    flat = [v for b in blocks for v in b[1]]
+    iovs = (FileIov * max(len(flat), 1))()
+    for k, v in enumerate(flat):
+        if isinstance(v, np.ndarray):
+            iovs[k] = FileIov(0, 0, v.ctypes.data, v.nbytes)
+        elif isinstance(v, tuple):
+            iovs[k] = FileIov(0, 0, None, int(v[1]))
+        else:
+            iovs[k] = FileIov(0, 1, 1, int(v))   # ignored: the base is never touched
+    return fn(os.fsencode(path), int(bsz), _p(blkids), _p(sz), _p(counts), C.addressof(iovs), n)
+
+
+def file_put(path, bsz, blocks, sizes=None):
+    """LocalFileSdk::DoPut on host iovs (local_file_sdk.cc:262-364). Returns 0 / -1 invalid / -4 file I/O."""
+    return _file_call(lib().kvcm_ref_file_put, path, bsz, blocks, sizes)
+
+
+def file_get(path, bsz, blocks, sizes=None):
+    """LocalFileSdk::DoGet on host iovs (local_file_sdk.cc:161-260)."""
+    return _file_call(lib().kvcm_ref_file_get, path, bsz, blocks, sizes)
 
 
 # ---------------------------------------------------------------------------------------------- buffer check

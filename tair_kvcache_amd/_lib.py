@@ -26,6 +26,7 @@ OK = 0
 ERR_INVALID_ARG = -1
 ERR_ALIGNMENT = -2
 ERR_TOO_LARGE = -3
+ERR_IO = -4
 
 i32, i64, vp, sz = C.c_int32, C.c_int64, C.c_void_p, C.c_size_t
 
@@ -67,6 +68,10 @@ SIGNATURES = {
     "kvcm_hip_mask_to_indices": (i32, [vp, vp, i64, vp, i64, vp, vp, vp]),
     "kvcm_hip_iov_crc32": (i32, [vp, i32, vp, sz, vp]),
     "kvcm_blocks_hash_from_crcs": (i32, [vp, i64, i32, vp]),
+    "kvcm_file_store_create": (i32, [i64, i64, i32, C.POINTER(vp)]),
+    "kvcm_file_store_destroy": (None, [vp]),
+    "kvcm_file_store_put": (i32, [vp, C.c_char_p, vp, vp, vp, vp, i32]),
+    "kvcm_file_store_get": (i32, [vp, C.c_char_p, vp, vp, vp, vp, i32]),
 }
 
 _lock = threading.Lock()

@@ -7,7 +7,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libkvcm_hip.so")
-SOURCES = ["kvcm_copy.hip", "kvcm_hash.hip", "kvcm_select.hip"]
+SOURCES = ["kvcm_copy.hip", "kvcm_hash.hip", "kvcm_select.hip", "kvcm_file.hip"]
 
 
 def hipcc_command(out=LIB_PATH):

@@ -17,9 +17,11 @@ class MemoryType(enum.IntEnum):
 class ClientErrorCode(enum.IntEnum):
     ER_OK = 0
     ER_INVALID_PARAMS = 3
+    ER_INVALID_SDKBACKEND_CONFIG = 8
     ER_SDK_TIMEOUT = 100
     ER_SDKREAD_ERROR = 104
     ER_SDKWRITE_ERROR = 105
+    ER_SDKALLOC_ERROR = 106
     ER_INVALID_LOCAL_BUFFERS = 108
     ER_FILE_IO_ERROR = 111
 

@@ -510,6 +510,8 @@ const char *kvcm_hip_error_string(int32_t code) {
             return "misaligned address or stride";
         case KVCM_ERR_TOO_LARGE:
             return "size exceeds the launch geometry";
+        case KVCM_ERR_IO:
+            return "file input/output error";
         default:
             return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown kvcm error";
     }
