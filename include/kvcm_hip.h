@@ -11,11 +11,13 @@
  * Conventions
  *   - every pointer whose name starts with d_ is DEVICE memory, readable/writable by kernels on the
  *     current HIP device; everything else is host memory;
- *   - all entry points are asynchronous on `stream` (a hipStream_t passed as void*; NULL = null stream),
+ *   - all kvcm_hip_* entry points are asynchronous on `stream` (a hipStream_t passed as void*; NULL = null stream),
  *     never synchronise, never allocate, never switch device, and keep no global mutable state, so they
  *     can be called concurrently from many host threads (the reference calls its kernels from a
  *     32-thread pool: kv_cache_manager/py_connector/vllm/data_transfer.py:80-93);
  *   - device buffers passed in must stay alive until `stream` has executed the call;
+ *   - the kvcm_file_store_* family at the end is host-side file I/O: it blocks, and it owns streams and pinned
+ *     buffers between create and destroy;
  *   - return value: 0 = OK, negative = KVCM_ERR_* (argument rejected, nothing launched),
  *     positive = a hipError_t reported by the launch.
  *
