@@ -160,4 +160,93 @@ inline std::vector<int64_t> GetBlocksHash(const std::vector<kvcm_iov_device> &io
     return out;
 }
 
+// In-batch duplicate detection on block keys: (*first_idx)[i] = smallest j with keys[j] == keys[i]. The batched,
+// client-side counterpart of the manager's per-request filter (kv_cache_manager/manager/cache_manager.cc:589-635).
+inline int32_t FirstOccurrence(const KeyVector &keys, std::vector<int32_t> *first_idx, hipStream_t stream = nullptr) {
+    if (!first_idx) {
+        return KVCM_ERR_INVALID_ARG;
+    }
+    first_idx->assign(keys.size(), 0);
+    if (keys.empty()) {
+        return KVCM_OK;
+    }
+    const int64_t n = static_cast<int64_t>(keys.size());
+    const int64_t ws_bytes = kvcm_hip_first_occurrence_workspace_bytes(n);
+    if (ws_bytes < 0) {
+        return static_cast<int32_t>(ws_bytes);
+    }
+    detail::DeviceArray<int64_t> d_keys(keys.size());
+    detail::DeviceArray<int32_t> d_first(keys.size()), d_ws(static_cast<size_t>(ws_bytes / 4));
+    if (!d_keys.ptr || !d_first.ptr || !d_ws.ptr) {
+        return static_cast<int32_t>(hipErrorOutOfMemory);
+    }
+    hipError_t e = hipMemcpyAsync(d_keys.ptr, keys.data(), keys.size() * 8, hipMemcpyHostToDevice, stream);
+    if (e != hipSuccess) {
+        return static_cast<int32_t>(e);
+    }
+    const int32_t rc = kvcm_hip_first_occurrence(d_keys.ptr, n, d_ws.ptr, ws_bytes, d_first.ptr, nullptr, stream);
+    if (rc != KVCM_OK) {
+        (void)hipStreamSynchronize(stream);
+        return rc;
+    }
+    e = hipMemcpyAsync(first_idx->data(), d_first.ptr, keys.size() * 4, hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) {
+        e = hipStreamSynchronize(stream);
+    }
+    return e == hipSuccess ? KVCM_OK : static_cast<int32_t>(e);
+}
+
+// Block files with the reference's layout (kv_cache_manager/client/src/internal/sdk/local_file_sdk.cc:161-364):
+// owns a kvcm_file_store. One BlockBuffer per block, as kv_cache_manager/client/include/common.h:116-118.
+struct BlockBuffer {
+    std::vector<kvcm_iov> iovs;
+};
+
+class LocalFileStore {
+public:
+    explicit LocalFileStore(int64_t byte_size_per_block, int64_t bounce_bytes = 0, bool sync_on_put = true) {
+        if (kvcm_file_store_create(byte_size_per_block, bounce_bytes, sync_on_put ? 1 : 0, &store_) != KVCM_OK) {
+            store_ = nullptr;
+        }
+        size_ = static_cast<uint64_t>(byte_size_per_block);
+    }
+    ~LocalFileStore() { kvcm_file_store_destroy(store_); }
+    LocalFileStore(const LocalFileStore &) = delete;
+    LocalFileStore &operator=(const LocalFileStore &) = delete;
+    bool Valid() const { return store_ != nullptr; }
+
+    // All blocks go to the one file `path`; blkids[b] and uri_sizes[b] are the URI parameters of block b
+    // (uri_sizes empty = the store's block size).
+    int32_t Put(const char *path, const std::vector<uint64_t> &blkids, const std::vector<BlockBuffer> &buffers,
+                const std::vector<uint64_t> &uri_sizes = {}) {
+        return Call(kvcm_file_store_put, path, blkids, buffers, uri_sizes);
+    }
+    int32_t Get(const char *path, const std::vector<uint64_t> &blkids, const std::vector<BlockBuffer> &buffers,
+                const std::vector<uint64_t> &uri_sizes = {}) {
+        return Call(kvcm_file_store_get, path, blkids, buffers, uri_sizes);
+    }
+
+private:
+    template <typename Fn>
+    int32_t Call(Fn fn, const char *path, const std::vector<uint64_t> &blkids, const std::vector<BlockBuffer> &buffers,
+                 const std::vector<uint64_t> &uri_sizes) {
+        if (!store_ || blkids.size() != buffers.size() || (!uri_sizes.empty() && uri_sizes.size() != blkids.size()) ||
+            blkids.size() > static_cast<size_t>(INT32_MAX)) {
+            return KVCM_ERR_INVALID_ARG;
+        }
+        std::vector<uint64_t> sizes = uri_sizes.empty() ? std::vector<uint64_t>(blkids.size(), size_) : uri_sizes;
+        std::vector<int32_t> counts;
+        std::vector<kvcm_iov> flat;
+        for (const BlockBuffer &b : buffers) {
+            counts.push_back(static_cast<int32_t>(b.iovs.size()));
+            flat.insert(flat.end(), b.iovs.begin(), b.iovs.end());
+        }
+        return fn(store_, path, blkids.data(), sizes.data(), counts.data(), flat.data(),
+                  static_cast<int32_t>(blkids.size()));
+    }
+
+    kvcm_file_store *store_ = nullptr;
+    uint64_t size_ = 0;
+};
+
 }  // namespace kvcm

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <random>
 #include <string>
@@ -173,6 +174,87 @@ static void test_gather_scatter_c_abi() {
     (void)hipStreamDestroy(stream);
 }
 
+// The reference's own GPU unit test of the local-file SDK restated on this library
+// (kv_cache_manager/client/src/internal/sdk/test/local_file_sdk_test.cc:97-172): two device iovs of one 1024-byte
+// block, a URI size that does not match refused, the bytes read back into fresh device memory.
+static void test_local_file_put_get_with_gpu() {
+    const char *test_data = "this is local file test";
+    const char *test_data_2 = "and this is another local file test";
+    const size_t len1 = std::strlen(test_data), len2 = std::strlen(test_data_2);
+    std::string host_put = std::string(test_data) + test_data_2;
+    char tmpl[] = "/tmp/kvcm_cpp_XXXXXX";
+    const char *dir = mkdtemp(tmpl);
+    EXPECT(dir != nullptr);
+    const std::string path = std::string(dir ? dir : "/tmp") + "/local_file/test_gpu.txt";
+
+    char *gpu_put = nullptr, *gpu_get = nullptr;
+    EXPECT(hipMalloc(reinterpret_cast<void **>(&gpu_put), len1 + len2) == hipSuccess);
+    EXPECT(hipMalloc(reinterpret_cast<void **>(&gpu_get), len1 + len2) == hipSuccess);
+    EXPECT(hipMemcpy(gpu_put, host_put.data(), len1 + len2, hipMemcpyHostToDevice) == hipSuccess);
+    EXPECT(hipMemset(gpu_get, 0, len1 + len2) == hipSuccess);
+
+    kvcm::LocalFileStore sdk(1024);
+    EXPECT(sdk.Valid());
+    kvcm::BlockBuffer buf;
+    buf.iovs.push_back(kvcm_iov{KVCM_MEMORY_GPU, 0, gpu_put, len1});
+    buf.iovs.push_back(kvcm_iov{KVCM_MEMORY_GPU, 0, gpu_put + len1, len2});
+    EXPECT(sdk.Put(path.c_str(), {0}, {buf}, {1023}) == KVCM_ERR_INVALID_ARG);
+    EXPECT(sdk.Put(path.c_str(), {0}, {buf}) == KVCM_OK);
+
+    // the file is what the reference's DoPut leaves (restated in the oracle, host iovs)
+    const std::string ref_path = std::string(dir ? dir : "/tmp") + "/reference.bin";
+    const uint64_t blkid = 0, size = 1024;
+    const int32_t count = 2;
+    kvcm_ref_fiov fiovs[2] = {{0, 0, const_cast<char *>(host_put.data()), len1},
+                              {0, 0, const_cast<char *>(host_put.data()) + len1, len2}};
+    EXPECT(kvcm_ref_file_put(ref_path.c_str(), 1024, &blkid, &size, &count, fiovs, 1) == 0);
+    auto slurp = [](const std::string &p) {
+        std::string out;
+        if (FILE *f = std::fopen(p.c_str(), "rb")) {
+            char chunk[4096];
+            size_t got;
+            while ((got = std::fread(chunk, 1, sizeof chunk, f)) > 0) {
+                out.append(chunk, got);
+            }
+            std::fclose(f);
+        }
+        return out;
+    };
+    EXPECT(slurp(path).size() == 1024 && slurp(path) == slurp(ref_path));
+
+    kvcm::BlockBuffer gbuf;
+    gbuf.iovs.push_back(kvcm_iov{KVCM_MEMORY_GPU, 0, gpu_get, len1});
+    gbuf.iovs.push_back(kvcm_iov{KVCM_MEMORY_GPU, 0, gpu_get + len1, len2});
+    EXPECT(sdk.Get(path.c_str(), {0}, {gbuf}, {1023}) == KVCM_ERR_INVALID_ARG);
+    EXPECT(sdk.Get(ref_path.c_str(), {0}, {gbuf}) == KVCM_OK);
+    std::string host_get(len1 + len2, '\0');
+    EXPECT(hipMemcpy(&host_get[0], gpu_get, len1 + len2, hipMemcpyDeviceToHost) == hipSuccess);
+    EXPECT(host_get == host_put);
+    EXPECT(sdk.Get((path + ".missing").c_str(), {0}, {gbuf}) == KVCM_ERR_IO);
+    (void)hipFree(gpu_put);
+    (void)hipFree(gpu_get);
+}
+
+static void test_first_occurrence() {
+    std::mt19937_64 rng(99);
+    std::vector<int64_t> base(700), keys(5000);
+    for (auto &b : base) {
+        b = static_cast<int64_t>(rng());
+    }
+    for (auto &k : keys) {
+        k = base[rng() % base.size()];
+    }
+    keys[7] = INT64_MIN;
+    keys[4999] = INT64_MIN;
+    std::vector<int32_t> got, want(keys.size());
+    EXPECT(kvcm::FirstOccurrence(keys, &got) == KVCM_OK);
+    EXPECT(kvcm_ref_first_occurrence(keys.data(), static_cast<int64_t>(keys.size()), want.data(), nullptr) == 0);
+    EXPECT(got == want);
+    EXPECT(got[4999] == 7);
+    std::vector<int32_t> none;
+    EXPECT(kvcm::FirstOccurrence({}, &none) == KVCM_OK && none.empty());
+}
+
 int main() {
     int n = 0;
     if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
@@ -183,6 +265,8 @@ int main() {
     test_blocks_hash();
     test_gen_key_vector();
     test_gather_scatter_c_abi();
+    test_local_file_put_get_with_gpu();
+    test_first_occurrence();
     std::printf("%d checks, %d failed\n", g_run, g_failed);
     return g_failed == 0 ? 0 : 1;
 }
