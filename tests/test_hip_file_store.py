@@ -218,3 +218,38 @@ def test_save_to_files_then_load_through_the_transfer_manager(oracle, tmp_path):
     mgr.shutdown()
     mgr2.shutdown()
     client.close()
+
+
+def test_sglang_page_first_pool_on_the_device(oracle, tmp_path):
+    """The page_first_direct pool of py_connector/sglang/test.py:146-151 kept in HBM: two device iovs per block, no
+    gather, files equal to the oracle's DoPut of the same bytes."""
+    from tair_kvcache_amd import client_types as ct
+    from tair_kvcache_amd.local_file_sdk import LocalFileTransferClient
+    pages, layers, page_size, heads, dim = 40, 4, 64, 8, 128
+    rng = np.random.default_rng(21)
+    pool = rng.integers(0, 65536, size=(2, pages, layers, page_size, heads, dim), dtype=np.uint16)
+    d_pool = dev(pool)
+    piece = layers * page_size * heads * dim * 2
+    bsz = 2 * piece
+    client = LocalFileTransferClient(bsz, sync_on_put=False)
+    page_ids = rng.permutation(pages)[:16].tolist()
+
+    def buffers(t):
+        return [ct.BlockBuffer(iovs=[ct.Iov(type=ct.MemoryType.GPU, base=t[kv, pg].data_ptr(), size=piece, ignore=False)
+                                     for kv in (0, 1)]) for pg in page_ids]
+
+    path = str(tmp_path / "hicache" / "blocks")
+    uris = [_uri(path, i, bsz) for i in range(len(page_ids))]
+    code, _ = client.SaveKvCaches(uris, buffers(d_pool))
+    assert code == ct.ClientErrorCode.ER_OK
+    theirs = str(tmp_path / "oracle_blocks")
+    blocks = [(i, [pool[0, pg].reshape(-1).view(np.uint8), pool[1, pg].reshape(-1).view(np.uint8)])
+              for i, pg in enumerate(page_ids)]
+    assert oracle.file_put(theirs, bsz, blocks) == 0
+    assert open(path, "rb").read() == open(theirs, "rb").read()
+    back = torch.zeros_like(d_pool)
+    assert client.LoadKvCaches([_uri(theirs, i, bsz) for i in range(len(page_ids))], buffers(back)) == 0
+    got = host(back, np.uint16)
+    for pg in range(pages):
+        assert (got[:, pg] == (pool[:, pg] if pg in page_ids else 0)).all()
+    client.close()

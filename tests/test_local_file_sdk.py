@@ -193,3 +193,44 @@ def test_blocks_are_grouped_by_file(tmp_path):
     code, actual = client.SaveKvCaches([_uri(a, 0, bsz + 1)], [ct.BlockBuffer(iovs=[_iov(data[0])])])
     assert code == EC.ER_SDKWRITE_ERROR and actual == []
     client.close()
+
+
+def test_sglang_page_first_pool_goes_to_files_without_a_gather(oracle, tmp_path):
+    """SGLang's host pool in the page_first_direct layout, (2, pages, layers, page_size, heads, dim)
+    (py_connector/sglang/test.py:48,146-151): a page's K and V are one contiguous piece each, so the connector hands
+    the transfer client two iovs per block (_prepare_buffers, sglang/connector.py:426-440) and nothing is gathered.
+    The pool is filled as the reference's test fills it (value = token index)."""
+    pages, layers, page_size, heads, dim = 12, 3, 8, 2, 16
+    pool = np.zeros((2, pages, layers, page_size, heads, dim), dtype=np.uint16)
+    for i in range(pages * page_size):
+        pool[:, i // page_size, :, i % page_size] = i
+    piece = layers * page_size * heads * dim * 2          # bytes of one page's K (or V)
+    bsz = 2 * piece                                       # location_spec_size = size per token * page_size
+    client = LocalFileTransferClient(bsz)
+    page_ids = [7, 0, 3, 11]
+
+    def buffers(arr):
+        out = []
+        for pg in page_ids:
+            iovs = [ct.Iov(type=ct.MemoryType.CPU, base=arr[kv, pg].ctypes.data, size=piece, ignore=False)
+                    for kv in (0, 1)]
+            out.append(ct.BlockBuffer(iovs=iovs))
+        return out
+
+    path = str(tmp_path / "hicache" / "blocks")
+    uris = [_uri(path, i, bsz) for i in range(len(page_ids))]
+    code, _ = client.SaveKvCaches(uris, buffers(pool))
+    assert code == EC.ER_OK
+    raw = np.frombuffer(open(path, "rb").read(), dtype=np.uint16).reshape(len(page_ids), 2, layers, page_size, heads, dim)
+    for i, pg in enumerate(page_ids):
+        assert (raw[i, 0] == pool[0, pg]).all() and (raw[i, 1] == pool[1, pg]).all()
+    theirs = str(tmp_path / "oracle_blocks")
+    blocks = [(i, [pool[0, pg].reshape(-1).view(np.uint8), pool[1, pg].reshape(-1).view(np.uint8)])
+              for i, pg in enumerate(page_ids)]
+    assert oracle.file_put(theirs, bsz, blocks) == 0
+    assert open(path, "rb").read() == open(theirs, "rb").read()
+    back = np.zeros_like(pool)
+    assert client.LoadKvCaches(uris, buffers(back)) == EC.ER_OK
+    for pg in range(pages):
+        assert (back[:, pg] == (pool[:, pg] if pg in page_ids else 0)).all()
+    client.close()
