@@ -253,3 +253,35 @@ def test_sglang_page_first_pool_on_the_device(oracle, tmp_path):
     for pg in range(pages):
         assert (got[:, pg] == (pool[:, pg] if pg in page_ids else 0)).all()
     client.close()
+
+
+def test_trtllm_block_major_pool_on_the_device(oracle, tmp_path):
+    """TensorRT-LLM's pool is block-major, {blocks, layers, K|V, block_size} (py_connector/trtllm/connector.py:173-179):
+    a block is contiguous, the reference copies it to the host (`kv_cache_tensor[block_id].cpu()`, :261-279) and hands
+    over a host iov. Here the block leaves as one device iov and comes back the same way."""
+    from tair_kvcache_amd import client_types as ct
+    from tair_kvcache_amd.local_file_sdk import LocalFileTransferClient
+    blocks_n, layers, kv, block_elems = 64, 6, 2, 32 * 4 * 64   # tokens_per_block * heads * head_dim
+    rng = np.random.default_rng(22)
+    pool = rng.integers(0, 65536, size=(blocks_n, layers, kv, block_elems), dtype=np.uint16)
+    d_pool = dev(pool)
+    bsz = layers * kv * block_elems * 2                        # location_spec_size (:180)
+    client = LocalFileTransferClient(bsz, bounce_bytes=1 << 20, sync_on_put=False)
+    block_ids = rng.permutation(blocks_n)[:20].tolist()
+
+    def buffers(t):
+        return [ct.BlockBuffer(iovs=[ct.Iov(type=ct.MemoryType.GPU, base=t[b].data_ptr(), size=bsz, ignore=False)])
+                for b in block_ids]
+
+    path = str(tmp_path / "trt" / "blocks")
+    uris = [_uri(path, i, bsz) for i in range(len(block_ids))]
+    assert client.SaveKvCaches(uris, buffers(d_pool))[0] == ct.ClientErrorCode.ER_OK
+    theirs = str(tmp_path / "oracle_blocks")
+    assert oracle.file_put(theirs, bsz, [(i, [pool[b].reshape(-1).view(np.uint8)]) for i, b in enumerate(block_ids)]) == 0
+    assert open(path, "rb").read() == open(theirs, "rb").read()
+    back = torch.zeros_like(d_pool)
+    assert client.LoadKvCaches([_uri(theirs, i, bsz) for i in range(len(block_ids))], buffers(back)) == 0
+    got = host(back, np.uint16)
+    for b in range(blocks_n):
+        assert (got[b] == (pool[b] if b in block_ids else 0)).all()
+    client.close()
