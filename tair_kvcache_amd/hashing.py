@@ -56,6 +56,8 @@ def hash_tokens(tokens: torch.Tensor, block_size: int, token_offsets: Optional[t
         else:
             total = int(key_offsets[-1].item())
         keys = torch.empty(total, dtype=torch.int64, device=tokens.device)
+        if total == 0:  # no request holds a full block: nothing to launch (GenKeyVector returns an empty vector)
+            return keys, key_offsets
     fn = lib().kvcm_hip_hash_tokens if tokens.dtype == torch.int64 else lib().kvcm_hip_hash_tokens_i32
     rc = fn(ptr(tokens), ptr(off), R, int(block_size), int(seed), ptr(keys), ptr(key_offsets),
             stream_handle(tokens.device))
