@@ -311,6 +311,19 @@ int32_t kvcm_file_store_put(kvcm_file_store *store, const char *path, const uint
 int32_t kvcm_file_store_get(kvcm_file_store *store, const char *path, const uint64_t *blkids, const uint64_t *sizes,
                             const int32_t *iov_counts, const kvcm_iov *iovs, int32_t n_blocks);
 
+/*
+ * iovs <-> one contiguous host buffer (the I/O buffer a storage client reads from or writes into): the pieces lie back
+ * to back in the buffer in iov order; IGNORED iovs take no room in it (unlike in a block file).
+ * load = 0 packs the iovs into the buffer, load != 0 unpacks the buffer into the iovs. Device iovs are copied
+ * asynchronously on `stream` and the call returns after the stream has been synchronised, as the reference does; host
+ * iovs are memcpy'd. A pinned host buffer gives full-speed copies; a pageable one works.
+ * Replaces: Hf3fsUsrbioClient::CopyIovs  kv_cache_manager/client/src/internal/sdk/hf3fs_usrbio_client.cc:478-505
+ *           over Hf3fsCudaUtil            kv_cache_manager/client/src/internal/sdk/hf3fs_cuda_util.h:21-79.
+ * Returns KVCM_ERR_INVALID_ARG when the pieces do not fit into host_buffer_size (nothing is copied then).
+ */
+int32_t kvcm_copy_iovs(void *host_buffer, size_t host_buffer_size, const kvcm_iov *iovs, int32_t n, int32_t load,
+                       kvcm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

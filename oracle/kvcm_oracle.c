@@ -674,3 +674,23 @@ int32_t kvcm_ref_file_get(const char *path, int64_t bsz, const uint64_t *blkids,
     close(fd);
     return rc;
 }
+
+/* hf3fs_usrbio_client.cc:478-505 (CopyIovs) on host iovs: pieces back to back in the I/O buffer; an ignored iov is
+ * skipped WITHOUT advancing the offset (:484-486), a null base is not tested for there (the caller never passes one). */
+int64_t kvcm_ref_copy_iovs(void *host_buffer, const kvcm_ref_fiov *iovs, int32_t n, int32_t load) {
+    int64_t iov_offset = 0;
+    char *iov_base = (char *)host_buffer;
+    for (int32_t i = 0; i < n; i++) {
+        const kvcm_ref_fiov *iov = &iovs[i];
+        if (iov->ignore) {
+            continue;
+        }
+        if (load) {
+            memcpy(iov->base, iov_base + iov_offset, iov->size);
+        } else {
+            memcpy(iov_base + iov_offset, iov->base, iov->size);
+        }
+        iov_offset += (int64_t)iov->size;
+    }
+    return iov_offset;
+}

@@ -127,6 +127,10 @@ int32_t kvcm_ref_file_put(const char *path, int64_t bsz, const uint64_t *blkids,
 int32_t kvcm_ref_file_get(const char *path, int64_t bsz, const uint64_t *blkids, const uint64_t *sizes,
                           const int32_t *iov_counts, const kvcm_ref_fiov *iovs, int32_t n_blocks);
 
+/* Hf3fsUsrbioClient::CopyIovs on host iovs: kv_cache_manager/client/src/internal/sdk/hf3fs_usrbio_client.cc:478-505.
+ * Returns the number of bytes the iovs take in the buffer. */
+int64_t kvcm_ref_copy_iovs(void *host_buffer, const kvcm_ref_fiov *iovs, int32_t n, int32_t load);
+
 #ifdef __cplusplus
 }
 #endif

@@ -110,6 +110,8 @@ def lib():
         for name in ("kvcm_ref_file_put", "kvcm_ref_file_get"):
             getattr(L, name).restype = i32
             getattr(L, name).argtypes = [C.c_char_p, i64, vp, vp, vp, vp, i32]
+        L.kvcm_ref_copy_iovs.restype = i64
+        L.kvcm_ref_copy_iovs.argtypes = [vp, vp, i32, i32]
         L.kvcm_ref_first_occurrence.restype = i32
         L.kvcm_ref_first_occurrence.argtypes = [vp, i64, vp, vp]
         L.kvcm_ref_mask_to_indices.restype = i64
@@ -415,6 +417,15 @@ def file_put(path, bsz, blocks, sizes=None):
 def file_get(path, bsz, blocks, sizes=None):
     """LocalFileSdk::DoGet on host iovs (local_file_sdk.cc:161-260)."""
     return _file_call(lib().kvcm_ref_file_get, path, bsz, blocks, sizes)
+
+
+def copy_iovs(host_buffer, pieces, load):
+    """Hf3fsUsrbioClient::CopyIovs on host iovs (hf3fs_usrbio_client.cc:478-505). pieces: NumPy uint8 arrays, or an
+    int n for an ignored iov of n bytes. Returns the bytes used in host_buffer."""
+    iovs = (FileIov * max(len(pieces), 1))()
+    for k, v in enumerate(pieces):
+        iovs[k] = FileIov(0, 0, v.ctypes.data, v.nbytes) if isinstance(v, np.ndarray) else FileIov(0, 1, 1, int(v))
+    return lib().kvcm_ref_copy_iovs(host_buffer.ctypes.data, C.addressof(iovs), len(pieces), int(load))
 
 
 # ---------------------------------------------------------------------------------------------- buffer check

@@ -72,6 +72,7 @@ SIGNATURES = {
     "kvcm_file_store_destroy": (None, [vp]),
     "kvcm_file_store_put": (i32, [vp, C.c_char_p, vp, vp, vp, vp, i32]),
     "kvcm_file_store_get": (i32, [vp, C.c_char_p, vp, vp, vp, vp, i32]),
+    "kvcm_copy_iovs": (i32, [vp, sz, vp, i32, i32, vp]),
 }
 
 _lock = threading.Lock()

@@ -13,6 +13,7 @@
 // chunks, and the copy engine fills one bounce buffer while the host writes the other one out with pwrite (or, on
 // Get, pread fills one while the other is copied up). Host iovs are written and read in place.
 #include <errno.h>
+#include <string.h>
 #include <fcntl.h>
 #include <sys/stat.h>
 #include <unistd.h>
@@ -421,6 +422,56 @@ int32_t kvcm_file_store_get(kvcm_file_store *store, const char *path, const uint
     }
     close(fd);
     return rc;
+}
+
+int32_t kvcm_copy_iovs(void *host_buffer, size_t host_buffer_size, const kvcm_iov *iovs, int32_t n, int32_t load,
+                       kvcm_stream_t stream) {
+    if (n < 0 || (n > 0 && (!iovs || !host_buffer))) {
+        return KVCM_ERR_INVALID_ARG;
+    }
+    size_t total = 0;
+    for (int32_t i = 0; i < n; i++) {
+        if (iovs[i].ignore) {
+            continue;
+        }
+        if (iovs[i].type != KVCM_MEMORY_CPU && iovs[i].type != KVCM_MEMORY_GPU) {
+            return KVCM_ERR_INVALID_ARG;
+        }
+        if (iovs[i].size > host_buffer_size - total) {
+            return KVCM_ERR_INVALID_ARG;
+        }
+        total += iovs[i].size;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    char *buffer = static_cast<char *>(host_buffer);
+    size_t offset = 0;
+    bool device = false;
+    hipError_t e = hipSuccess;
+    for (int32_t i = 0; i < n && e == hipSuccess; i++) {
+        const kvcm_iov &iov = iovs[i];
+        if (iov.ignore) {
+            continue;
+        }
+        if (iov.base && iov.size > 0) {
+            if (iov.type == KVCM_MEMORY_GPU) {
+                device = true;
+                e = load ? hipMemcpyAsync(iov.base, buffer + offset, iov.size, hipMemcpyHostToDevice, s)
+                         : hipMemcpyAsync(buffer + offset, iov.base, iov.size, hipMemcpyDeviceToHost, s);
+            } else if (load) {
+                memcpy(iov.base, buffer + offset, iov.size);
+            } else {
+                memcpy(buffer + offset, iov.base, iov.size);
+            }
+        }
+        offset += iov.size;
+    }
+    if (device) {
+        hipError_t sync = hipStreamSynchronize(s);
+        if (e == hipSuccess) {
+            e = sync;
+        }
+    }
+    return kvcm::hip_code(e);
 }
 
 }  // extern "C"

@@ -3,6 +3,8 @@
     StandardUri              kv_cache_manager/common/standard_uri.cc:16-140
     LocalFileSdk             kv_cache_manager/client/src/internal/sdk/local_file_sdk.cc:61-364
                              (SplitByPath: kv_cache_manager/client/src/internal/sdk/sdk_interface.cc:5-17)
+    copy_iovs                Hf3fsUsrbioClient::CopyIovs
+                             kv_cache_manager/client/src/internal/sdk/hf3fs_usrbio_client.cc:478-505
     LocalFileTransferClient  the TransferClient surface the connector calls
                              (kv_cache_manager/client/include/transfer_client.h:19-21,
                               kv_cache_manager/client/src/transfer_client_impl.cc:119-161) over one LocalFileSdk
@@ -116,6 +118,19 @@ class StandardUri:
 class _Iov(C.Structure):
     """struct kvcm_iov."""
     _fields_ = [("type", C.c_uint8), ("ignore", C.c_uint8), ("base", C.c_void_p), ("size", C.c_size_t)]
+
+
+def copy_iovs(host_buffer_ptr: int, host_buffer_size: int, iovs, load: bool, stream_handle=None) -> int:
+    """iovs <-> one contiguous host buffer, pieces back to back, ignored iovs taking no room
+    (Hf3fsUsrbioClient::CopyIovs, kv_cache_manager/client/src/internal/sdk/hf3fs_usrbio_client.cc:478-505).
+    `iovs` are objects with type / base / size / ignore. Returns the library's code (0 = done and synchronised)."""
+    arr = (_Iov * max(len(iovs), 1))()
+    for k, iov in enumerate(iovs):
+        arr[k].type = int(iov.type)
+        arr[k].ignore = 1 if iov.ignore else 0
+        arr[k].base = int(iov.base) or None
+        arr[k].size = int(iov.size)
+    return lib().kvcm_copy_iovs(host_buffer_ptr, host_buffer_size, arr, len(iovs), 1 if load else 0, stream_handle)
 
 
 def _as_uri(u) -> StandardUri:

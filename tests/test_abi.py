@@ -21,7 +21,9 @@ def test_header_declares_the_expected_entry_points():
                  "kvcm_hip_paged_gather", "kvcm_hip_paged_scatter", "kvcm_hip_gather_ex", "kvcm_hip_scatter_ex",
                  "kvcm_hip_generate_blocks_idx", "kvcm_hip_iov_crc32", "kvcm_blocks_hash_from_crcs",
                  "kvcm_hip_first_occurrence", "kvcm_hip_first_occurrence_workspace_bytes",
-                 "kvcm_hip_mask_to_indices", "kvcm_hip_mask_to_indices_workspace_bytes"):
+                 "kvcm_hip_mask_to_indices", "kvcm_hip_mask_to_indices_workspace_bytes",
+                 "kvcm_file_store_create", "kvcm_file_store_destroy", "kvcm_file_store_put", "kvcm_file_store_get",
+                 "kvcm_copy_iovs"):
         assert must in names
 
 
@@ -39,7 +41,8 @@ def test_every_prototype_cites_the_reference():
     for anchor in ("cache_manager.cc:76-87", "hash_util.h:8-24", "trace_util.cc:47-56", "connector.py:397-415",
                    "batch_gather_scatter_helper.py:33-136", "batch_gather_scatter_helper.py:139-248",
                    "v1_connector.py:308-320", "sdk_buffer_check_util.cu:21-44", "sdk_buffer_check_util.cc:56-60",
-                   "v1_connector.py:835-850", "cache_manager.cc:589-635"):
+                   "v1_connector.py:835-850", "cache_manager.cc:589-635", "local_file_sdk.cc:68-85",
+                   "local_file_sdk.cc:161-260", "hf3fs_usrbio_client.cc:478-505", "common.h:102-110"):
         assert anchor in text, anchor
 
 

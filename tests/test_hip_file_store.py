@@ -285,3 +285,45 @@ def test_trtllm_block_major_pool_on_the_device(oracle, tmp_path):
     for b in range(blocks_n):
         assert (got[b] == (pool[b] if b in block_ids else 0)).all()
     client.close()
+
+
+def test_copy_iovs_with_device_pieces(oracle):
+    """The 3FS client's CopyIovs with device iovs: packed into a pinned I/O buffer and unpacked into fresh device
+    memory, against the oracle run on host copies."""
+    from tair_kvcache_amd import client_types as ct
+    from tair_kvcache_amd.local_file_sdk import copy_iovs
+    rng = np.random.default_rng(32)
+    arena = rng.integers(0, 256, size=1 << 20, dtype=np.uint8)
+    d_arena = torch.from_numpy(arena).cuda()
+    cuts = np.sort(rng.choice(np.arange(1, arena.size), size=9, replace=False)).tolist()
+    edges = [0] + cuts + [arena.size]
+    pieces, iovs = [], []
+    for j, (a, b) in enumerate(zip(edges[:-1], edges[1:])):
+        if j % 4 == 3:
+            pieces.append(b - a)
+            iovs.append(_giov(d_arena[a:b], ignore=True))
+        elif j % 4 == 1:
+            h = arena[a:b].copy()
+            pieces.append(h)
+            iovs.append(ct.Iov(type=ct.MemoryType.CPU, base=h.ctypes.data, size=h.nbytes, ignore=False))
+        else:
+            pieces.append(arena[a:b])
+            iovs.append(_giov(d_arena[a:b]))
+    need = sum(p.nbytes for p in pieces if isinstance(p, np.ndarray))
+    theirs = np.zeros(need, dtype=np.uint8)
+    assert oracle.copy_iovs(theirs, pieces, load=False) == need
+    pinned = torch.zeros(need, dtype=torch.uint8).pin_memory()
+    stream = torch.cuda.Stream()
+    assert copy_iovs(pinned.data_ptr(), need, iovs, load=False, stream_handle=stream.cuda_stream) == 0
+    assert (pinned.numpy() == theirs).all()
+    pageable = np.zeros(need, dtype=np.uint8)
+    assert copy_iovs(pageable.ctypes.data, need, iovs, load=False) == 0 and (pageable == theirs).all()
+    # unpack into a cleared arena: ignored ranges stay zero
+    d_arena.zero_()
+    assert copy_iovs(pinned.data_ptr(), need, iovs, load=True, stream_handle=stream.cuda_stream) == 0
+    got = d_arena.cpu().numpy()
+    for j, (a, b) in enumerate(zip(edges[:-1], edges[1:])):
+        if j % 4 == 3 or j % 4 == 1:
+            assert not got[a:b].any()
+        else:
+            assert (got[a:b] == arena[a:b]).all()

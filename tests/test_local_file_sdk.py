@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from tair_kvcache_amd import client_types as ct
-from tair_kvcache_amd.local_file_sdk import LocalFileSdk, LocalFileTransferClient, StandardUri
+from tair_kvcache_amd.local_file_sdk import LocalFileSdk, LocalFileTransferClient, StandardUri, copy_iovs
 
 EC = ct.ClientErrorCode
 
@@ -234,3 +234,38 @@ def test_sglang_page_first_pool_goes_to_files_without_a_gather(oracle, tmp_path)
     for pg in range(pages):
         assert (back[:, pg] == (pool[:, pg] if pg in page_ids else 0)).all()
     client.close()
+
+
+def test_copy_iovs_packs_like_the_oracle(oracle):
+    """iovs <-> one I/O buffer (the 3FS client's CopyIovs): ignored iovs take no room, pieces keep their order."""
+    rng = np.random.default_rng(31)
+    for trial in range(20):
+        pieces, iovs = [], []
+        for _ in range(int(rng.integers(0, 9))):
+            n = int(rng.integers(1, 3000))
+            if rng.random() < 0.25:
+                pieces.append(n)
+                iovs.append(ct.Iov(type=ct.MemoryType.CPU, base=1, size=n, ignore=True))
+            else:
+                a = rng.integers(0, 256, size=n, dtype=np.uint8)
+                pieces.append(a)
+                iovs.append(_iov(a))
+        need = sum(p.nbytes for p in pieces if isinstance(p, np.ndarray))
+        theirs = np.full(need + 64, 0xEE, dtype=np.uint8)
+        ours = np.full(need + 64, 0xEE, dtype=np.uint8)
+        assert oracle.copy_iovs(theirs, pieces, load=False) == need
+        assert copy_iovs(ours.ctypes.data, ours.nbytes, iovs, load=False) == 0
+        assert (ours == theirs).all() and (ours[need:] == 0xEE).all()
+        # and back out of the buffer into fresh arrays
+        outs = [np.zeros_like(p) if isinstance(p, np.ndarray) else p for p in pieces]
+        o_iovs = [_iov(o) if isinstance(o, np.ndarray) else ct.Iov(type=ct.MemoryType.CPU, base=1, size=o, ignore=True)
+                  for o in outs]
+        assert copy_iovs(theirs.ctypes.data, theirs.nbytes, o_iovs, load=True) == 0
+        for p, o in zip(pieces, outs):
+            if isinstance(p, np.ndarray):
+                assert (p == o).all()
+        # a buffer that is too small is refused before anything moves
+        if need > 1:
+            small = np.full(need - 1, 0xEE, dtype=np.uint8)
+            assert copy_iovs(small.ctypes.data, small.nbytes, iovs, load=False) == -1
+            assert (small == 0xEE).all()
