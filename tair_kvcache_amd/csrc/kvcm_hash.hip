@@ -201,10 +201,14 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
 // The chain wave's work on one tile: kTT steps from the lane's pre-added terms `a`, a key at every block
 // boundary. MASKED = some lane may have run out of tokens inside this tile (ragged batch); the common case of
 // equally long requests takes the unmasked path, which has no per-lane compare in it.
-template <int CHUNK, bool MASKED>
+// BS > 0 = the block size is this compile-time constant (a divisor or a multiple of the tile): the places where a key
+// is due are then known when the code is written, and the scalar bookkeeping (add, compare, branch per chunk: one
+// instruction slot in sixteen of the wave that sets the pace) disappears from the loop.
+template <int CHUNK, bool MASKED, int BS>
 __device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_t &h, int64_t t0, int64_t my_ntok,
                                          int32_t &since_key, int32_t block_size, int64_t *__restrict__ keys,
                                          int64_t &key_pos) {
+    static_assert(BS == 0 || (BS % CHUNK == 0 && (kTT % BS == 0 || BS % kTT == 0)), "block size fits the tiling");
 #pragma unroll
     for (int c = 0; c < kTT; c += CHUNK) {
         const bool active = !MASKED || (t0 + c) < my_ntok;
@@ -214,9 +218,19 @@ __device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_
                 h = chain_step(h, (s & 1) ? a[s / 2].y : a[s / 2].x);
             }
         }
-        since_key += CHUNK;
-        if (since_key == block_size) {
-            since_key = 0;
+        bool key_due;
+        if (BS == 0) {
+            since_key += CHUNK;
+            key_due = since_key == block_size;
+            if (key_due) {
+                since_key = 0;
+            }
+        } else if (BS <= kTT) {
+            key_due = (c + CHUNK) % BS == 0;  // tiles start on block boundaries
+        } else {
+            key_due = c + CHUNK == kTT && (t0 + kTT) % BS == 0;
+        }
+        if (key_due) {
             if (active) {
                 keys[key_pos] = static_cast<int64_t>(h);
             }
@@ -234,8 +248,8 @@ __device__ __forceinline__ void read_row(ulonglong2 (&a)[kTT / 2], const uint64_
 }
 
 // CHUNK = steps between two looks at the block boundary: 8 when block_size % 8 == 0 (a lane is then
-// active for whole chunks or not at all), otherwise 1.
-template <typename TokT, int CHUNK>
+// active for whole chunks or not at all), otherwise 1. BS = block size when it is 16, 32, 64 or 128, otherwise 0.
+template <typename TokT, int CHUNK, int BS>
 __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__restrict__ tokens,
                                                               const int64_t *__restrict__ token_offsets, int32_t R,
                                                               int32_t block_size, uint64_t seed,
@@ -263,8 +277,9 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     }
     __syncthreads();
 
+    // min over the requests that exist: the rows past R of the last workgroup do not make it "ragged"
     int64_t max_ntok = s_ntok[lane];
-    int64_t min_ntok = max_ntok;
+    int64_t min_ntok = r < R ? max_ntok : INT64_MAX;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         const int64_t hi_other = __shfl_xor(max_ntok, o);
@@ -307,12 +322,15 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     // A single wave issues one VALU instruction per ~4.8 cycles whether or not it depends on the previous one
     // (measured), so a step costs its instruction count; chain_step() is 6.
     uint64_t h = seed;
-    int64_t key_pos = 0;
-    if (r < R) {
-        key_pos = key_offsets ? key_offsets[r] : r * ((token_offsets[1] - token_offsets[0]) / block_size);
-    }
     int32_t since_key = 0;  // uniform: all lanes step in lockstep from token 0
     lds_barrier();
+    if (r >= R) {
+        // A lane without a request leaves here; the wave goes on without it (every workgroup has at least one request,
+        // so the wave still meets every barrier). This keeps the unmasked path, whose key stores are unconditional,
+        // usable when R is not a multiple of 64.
+        return;
+    }
+    int64_t key_pos = key_offsets ? key_offsets[r] : r * ((token_offsets[1] - token_offsets[0]) / block_size);
     ulonglong2 cur[kTT / 2], nxt[kTT / 2];
     read_row(cur, &s_tile[0][lane][0]);
     int ring = 0;
@@ -323,9 +341,9 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
             read_row(nxt, &s_tile[ring1][lane][0]);
         }
         if ((k + 1) * kTT <= min_ntok) {
-            run_tile<CHUNK, false>(cur, h, k * kTT, my_ntok, since_key, block_size, keys, key_pos);
+            run_tile<CHUNK, false, BS>(cur, h, k * kTT, my_ntok, since_key, block_size, keys, key_pos);
         } else {
-            run_tile<CHUNK, true>(cur, h, k * kTT, my_ntok, since_key, block_size, keys, key_pos);
+            run_tile<CHUNK, true, BS>(cur, h, k * kTT, my_ntok, since_key, block_size, keys, key_pos);
         }
         lds_barrier();
         if (k + 1 >= ntiles) {
@@ -336,9 +354,9 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
             read_row(cur, &s_tile[ring][lane][0]);
         }
         if ((k + 2) * kTT <= min_ntok) {
-            run_tile<CHUNK, false>(nxt, h, (k + 1) * kTT, my_ntok, since_key, block_size, keys, key_pos);
+            run_tile<CHUNK, false, BS>(nxt, h, (k + 1) * kTT, my_ntok, since_key, block_size, keys, key_pos);
         } else {
-            run_tile<CHUNK, true>(nxt, h, (k + 1) * kTT, my_ntok, since_key, block_size, keys, key_pos);
+            run_tile<CHUNK, true, BS>(nxt, h, (k + 1) * kTT, my_ntok, since_key, block_size, keys, key_pos);
         }
         lds_barrier();
     }
@@ -483,13 +501,23 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
     // test hook: take the loader path that a workgroup spanning >= 4 GiB of tokens would take
     const char *fg = std::getenv("KVCM_HASH_FORCE_GLOBAL_LOADS");
     const int32_t force_global = (fg && fg[0] == '1') ? 1 : 0;
-    if (block_size % 8 == 0) {
-        hipLaunchKernelGGL((hash_tokens_kernel<TokT, 8>), grid, dim3(kThreads), 0, stream, d_tokens, d_token_offsets, R,
-                           block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global);
+#define KVCM_LAUNCH_HASH(CHUNK, BS)                                                                                  \
+    hipLaunchKernelGGL((hash_tokens_kernel<TokT, CHUNK, BS>), grid, dim3(kThreads), 0, stream, d_tokens,            \
+                       d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
+    if (block_size == 16) {  // the engines' usual block sizes get kernels of their own
+        KVCM_LAUNCH_HASH(8, 16);
+    } else if (block_size == 32) {
+        KVCM_LAUNCH_HASH(8, 32);
+    } else if (block_size == 64) {
+        KVCM_LAUNCH_HASH(8, 64);
+    } else if (block_size == 128) {
+        KVCM_LAUNCH_HASH(8, 128);
+    } else if (block_size % 8 == 0) {
+        KVCM_LAUNCH_HASH(8, 0);
     } else {
-        hipLaunchKernelGGL((hash_tokens_kernel<TokT, 1>), grid, dim3(kThreads), 0, stream, d_tokens, d_token_offsets, R,
-                           block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global);
+        KVCM_LAUNCH_HASH(1, 0);
     }
+#undef KVCM_LAUNCH_HASH
     return launch_status();
 }
 
