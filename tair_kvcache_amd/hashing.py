@@ -37,7 +37,9 @@ def hash_tokens(tokens: torch.Tensor, block_size: int, token_offsets: Optional[t
 
     tokens: int64 or int32 device tensor, [R, L] (uniform lengths) or flat with token_offsets [R+1].
     Returns (keys, key_offsets): request r owns keys[key_offsets[r]:key_offsets[r+1]], len_r // block_size of
-    them (a trailing partial block yields no key, cache_manager.cc:78). Asynchronous on the current stream.
+    them (a trailing partial block yields no key, cache_manager.cc:78). Asynchronous on the current stream when
+    `keys` and `key_offsets` are passed in (or the batch is a 2-D tensor); otherwise the key offsets are computed with
+    torch and the total is read back to size `keys`, which costs a synchronisation (about 30 us on an idle MI355X).
     """
     require_cuda(tokens, "tokens")
     if tokens.dtype not in (torch.int64, torch.int32):
