@@ -23,6 +23,17 @@
  *         (py_connector/test/kernel/test_batch_gather_scatter.py:91-114,201-216), ramp-valued pools
  *         whose values name their own slot, scatter(gather) = identity, and canary guard bands.
  *   The trailer (per-block scale) interleave has no reference counterpart: brute force only.
+ *   kvcm_ref_first_occurrence / mask_to_indices
+ *       - brute force on small inputs, np.unique(return_index, return_inverse) on large ones, extreme signed keys;
+ *         the reference's parsing loop (py_connector/vllm/v1_connector.py:835-850) restated in Python, both branches.
+ *         first_occurrence has no reference counterpart (the manager filters per request, cache_manager.cc:589-635).
+ *   kvcm_ref_file_put / file_get
+ *       - the reference's own unit test at its own values (client/src/internal/sdk/test/local_file_sdk_test.cc:35-95);
+ *         the byte layout checked directly (blkid * size offsets, zero holes, a file never shrinks, spill into the
+ *         next block allowed, iovs past the end refused).
+ *   kvcm_ref_copy_iovs
+ *       - brute-force layout checks: ignored iovs take no room (hf3fs_usrbio_client.cc:484-486), order kept, canary
+ *         bytes after the last piece.
  */
 #define _GNU_SOURCE
 #include "kvcm_oracle.h"
