@@ -283,11 +283,13 @@ typedef struct kvcm_file_store kvcm_file_store;
  * byte_size_per_block must be positive. bounce_bytes = size of each pinned bounce buffer for device iovs (0 = 8 MiB);
  * they, and a stream, are created on the first call that meets a device iov, per concurrent caller (at most 64), and
  * live until the store is destroyed. sync_on_put != 0 ends every put with fdatasync, the counterpart of the
- * reference's msync(MS_SYNC) (:362). A store may be used from many threads at once. This family of entry points does
- * allocate and does block: it is file I/O.
+ * reference's msync(MS_SYNC) (:362). io_threads (0 = 4, at most 32) = threads that share the device iovs of ONE
+ * get, each with its own stream and buffers: a single thread is bound by pread, not by the link (a put stays on the
+ * calling thread: more writers to one new file gain nothing inside the kernel). A store may be used from many threads
+ * at once. This family of entry points does allocate and does block: it is file I/O.
  */
 int32_t kvcm_file_store_create(int64_t byte_size_per_block, int64_t bounce_bytes, int32_t sync_on_put,
-                               kvcm_file_store **out);
+                               int32_t io_threads, kvcm_file_store **out);
 void kvcm_file_store_destroy(kvcm_file_store *store);
 
 /*

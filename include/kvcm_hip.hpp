@@ -204,8 +204,10 @@ struct BlockBuffer {
 
 class LocalFileStore {
 public:
-    explicit LocalFileStore(int64_t byte_size_per_block, int64_t bounce_bytes = 0, bool sync_on_put = true) {
-        if (kvcm_file_store_create(byte_size_per_block, bounce_bytes, sync_on_put ? 1 : 0, &store_) != KVCM_OK) {
+    explicit LocalFileStore(int64_t byte_size_per_block, int64_t bounce_bytes = 0, bool sync_on_put = true,
+                            int32_t io_threads = 0) {
+        if (kvcm_file_store_create(byte_size_per_block, bounce_bytes, sync_on_put ? 1 : 0, io_threads, &store_) !=
+            KVCM_OK) {
             store_ = nullptr;
         }
         size_ = static_cast<uint64_t>(byte_size_per_block);

@@ -68,7 +68,7 @@ SIGNATURES = {
     "kvcm_hip_mask_to_indices": (i32, [vp, vp, i64, vp, i64, vp, vp, vp]),
     "kvcm_hip_iov_crc32": (i32, [vp, i32, vp, sz, vp]),
     "kvcm_blocks_hash_from_crcs": (i32, [vp, i64, i32, vp]),
-    "kvcm_file_store_create": (i32, [i64, i64, i32, C.POINTER(vp)]),
+    "kvcm_file_store_create": (i32, [i64, i64, i32, i32, C.POINTER(vp)]),
     "kvcm_file_store_destroy": (None, [vp]),
     "kvcm_file_store_put": (i32, [vp, C.c_char_p, vp, vp, vp, vp, i32]),
     "kvcm_file_store_get": (i32, [vp, C.c_char_p, vp, vp, vp, vp, i32]),

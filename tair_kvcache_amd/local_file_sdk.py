@@ -145,14 +145,19 @@ class LocalFileSdk:
         self._store = None
         self._byte_size_per_block = 0
 
-    def Init(self, byte_size_per_block, bounce_bytes: int = 0, sync_on_put: bool = True):
-        """Returns ER_INVALID_SDKBACKEND_CONFIG (8) for a missing or non-positive block size (local_file_sdk.cc:70-78)."""
+    def Init(self, byte_size_per_block, bounce_bytes: int = 0, sync_on_put: bool = True, io_threads: int = 0):
+        """Returns ER_INVALID_SDKBACKEND_CONFIG (8) for a missing or non-positive block size (local_file_sdk.cc:70-78),
+        and for a negative bounce size or more than 32 I/O threads. `io_threads` (0 = 4) is how many threads share the
+        device iovs of one Get."""
+        bad_config = getattr(self._cm.ClientErrorCode, "ER_INVALID_SDKBACKEND_CONFIG", 8)
         if byte_size_per_block is None or int(byte_size_per_block) <= 0:
-            return getattr(self._cm.ClientErrorCode, "ER_INVALID_SDKBACKEND_CONFIG", 8)
+            return bad_config
         self.close()
         handle = C.c_void_p()
         rc = lib().kvcm_file_store_create(int(byte_size_per_block), int(bounce_bytes), int(bool(sync_on_put)),
-                                          C.byref(handle))
+                                          int(io_threads), C.byref(handle))
+        if rc == _lib.ERR_INVALID_ARG:
+            return bad_config
         _lib.check(rc, "kvcm_file_store_create")
         self._store = handle
         self._byte_size_per_block = int(byte_size_per_block)
@@ -227,10 +232,10 @@ class LocalFileTransferClient:
     """SaveKvCaches / LoadKvCaches over block files; what `DataTransferManager` needs from a transfer client."""
 
     def __init__(self, byte_size_per_block: int, client_module=client_types, bounce_bytes: int = 0,
-                 sync_on_put: bool = True):
+                 sync_on_put: bool = True, io_threads: int = 0):
         self._cm = client_module
         self._sdk = LocalFileSdk(client_module)
-        code = self._sdk.Init(byte_size_per_block, bounce_bytes, sync_on_put)
+        code = self._sdk.Init(byte_size_per_block, bounce_bytes, sync_on_put, io_threads)
         if code != client_module.ClientErrorCode.ER_OK:
             raise ValueError(f"LocalFileSdk.Init failed with code {int(code)}")
 

@@ -133,6 +133,45 @@ def test_large_merged_run_of_staging_slots(oracle, tmp_path):
     sdk.close()
 
 
+def test_helper_threads_share_one_get(oracle, tmp_path):
+    """A Get of many chunks is split among the store's helper threads: every split (1, 2, 3, 8 and the maximum of 32
+    threads; 38 chunks of an odd size, so the ranges are ragged and the last chunk is short) reads the same bytes, a
+    second Get reuses the started helpers, and a Get from three callers at once divides them."""
+    from tair_kvcache_amd import client_types as ct
+    from tair_kvcache_amd.local_file_sdk import LocalFileSdk
+    EC = ct.ClientErrorCode
+    bsz, n, bounce = 100_000, 37, 99_993  # the 3.7 MB run of slots is one segment of 37 full chunks + 259 bytes
+    rng = np.random.default_rng(12)
+    data = rng.integers(0, 256, size=n * bsz, dtype=np.uint8)
+    theirs = str(tmp_path / "helpers.bin")
+    assert oracle.file_put(theirs, bsz, [(i, [data[i * bsz:(i + 1) * bsz]]) for i in range(n)]) == 0
+    d = torch.from_numpy(data).cuda()
+    uris = [_uri(theirs, i, bsz) for i in range(n)]
+    for io in (1, 2, 3, 8, 32):
+        sdk = LocalFileSdk()
+        assert sdk.Init(bsz, bounce_bytes=bounce, sync_on_put=False, io_threads=io) == EC.ER_OK
+        for _ in range(2):
+            back = torch.zeros_like(d)
+            bufs = [ct.BlockBuffer(iovs=[_giov(back[i * bsz:(i + 1) * bsz])]) for i in range(n)]
+            assert sdk.Get(uris, bufs) == EC.ER_OK
+            assert torch.equal(back, d), io
+        backs = [torch.zeros_like(d) for _ in range(3)]
+        codes = [None] * 3
+
+        def reader(k):
+            torch.cuda.set_device(0)
+            bufs = [ct.BlockBuffer(iovs=[_giov(backs[k][i * bsz:(i + 1) * bsz])]) for i in range(n)]
+            codes[k] = sdk.Get(uris, bufs)
+
+        threads = [threading.Thread(target=reader, args=(k,)) for k in range(3)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(120)
+        assert codes == [EC.ER_OK] * 3 and all(torch.equal(b, d) for b in backs), io
+        sdk.close()
+
+
 def test_many_threads_share_one_store(oracle, tmp_path):
     """The connector calls its transfer client from a thread pool: every caller gets its own stream and buffers."""
     from tair_kvcache_amd import client_types as ct

@@ -55,6 +55,8 @@ def test_init_like_the_reference():
     sdk = LocalFileSdk()
     assert sdk.Init(None) == EC.ER_INVALID_SDKBACKEND_CONFIG
     assert sdk.Init(-1) == EC.ER_INVALID_SDKBACKEND_CONFIG
+    assert sdk.Init(1024, io_threads=33) == EC.ER_INVALID_SDKBACKEND_CONFIG
+    assert sdk.Init(1024, io_threads=-1) == EC.ER_INVALID_SDKBACKEND_CONFIG
     assert sdk.Init(1024) == EC.ER_OK
     sdk.close()
 
