@@ -8,15 +8,15 @@
 // Design (gfx950, wave64): a workgroup owns 64 requests and is role-split.
 //   wave 0      "chain wave": lane = request. Keeps the state in VGPRs and does nothing but the recurrence,
 //               reading pre-added terms a = v + C from LDS (one ds_read_b128 per 2 steps, prefetched a whole
-//               tile ahead into a second register set). A single wave issues about one instruction per 4.8
-//               cycles whether or not it depends on the previous one (measured), so every instruction removed
-//               from this wave shortens the critical path of all 64 chains: the step is 6 instructions.
+//               tile ahead into a second register set). A lone wave issues a dependent VALU instruction 3.5-4 ns
+//               after its producer and independent ones 1.75 ns apart (measured), so the step is written for
+//               depth: three dependent levels, 5 instructions (see chain_step).
 //   waves 1..3  "loader waves": stream the 64 requests' tokens from HBM in [64 requests x 64 tokens] tiles with
 //               16-byte buffer loads (512-byte row segments), add C, and write them transposed into a 3-slot LDS
 //               ring. Each loader wave owns every third tile and keeps its loads in flight for about three
 //               tile periods, so HBM latency stays off the chain.
 // Roofline: HBM for many requests (8*block_size + 8 bytes per key); for few requests the bound is the
-// instruction issue rate of the chain wave, which no amount of bandwidth removes.
+// dependent-instruction latency of the chain wave, which no amount of bandwidth removes.
 #include "kvcm_internal.h"
 
 #include <cstdlib>
@@ -54,14 +54,18 @@ __device__ __forceinline__ void lds_barrier() {
 }
 
 // One step of the recurrence with the token term pre-added (a = v + C): h ^= a + (h << 12) + sar(h, 32).
-// Six single-issue VALU instructions: v_lshlrev_b64, v_ashrrev_i64, 2 x v_lshl_add_u64, 2 x v_xor_b32. The
-// arithmetic shift is written as the 64-bit instruction on purpose: left to itself the compiler splits sar(h, 32)
-// into v_ashrrev_i32 + v_mov_b32 (the pair {hi, sign} must be rebuilt in an even-aligned register pair), one
-// instruction more, and on a wave that is bound by instruction issue every instruction is 1/7 of the run time.
+// The wave that sets the pace is bound by the LATENCY of dependent VALU instructions (3.5-4 ns each, whatever the
+// instruction; measured on a lone wave), so what counts is the depth of the dependence chain, not the instruction
+// count. sar(h, 32) is the sign-extended upper half, and v_mad_i64_i32 (hi * 1 + a) adds it to `a` in ONE
+// instruction that needs only the upper half of h; the shift runs beside it, and the step is three levels deep:
+// {v_mad_i64_i32 | v_lshlrev_b64} -> v_lshl_add_u64 -> 2 x v_xor_b32 (10.9 ns per step against 12.4 ns for the
+// four-level form shift -> add -> add -> xor).
 __device__ __forceinline__ uint64_t chain_step(uint64_t h, uint64_t a) {
-    uint64_t sar;
-    asm("v_ashrrev_i64 %0, 32, %1" : "=v"(sar) : "v"(h));
-    return h ^ (a + (h << 12) + sar);
+    uint64_t a_plus_sar, carry_out;
+    asm("v_mad_i64_i32 %0, %1, %2, 1, %3"
+        : "=v"(a_plus_sar), "=s"(carry_out)
+        : "v"(static_cast<uint32_t>(h >> 32)), "v"(a));
+    return h ^ (a_plus_sar + (h << 12));
 }
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -319,8 +323,6 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     }
 
     // -------------------------------------------------------------------- chain wave
-    // A single wave issues one VALU instruction per ~4.8 cycles whether or not it depends on the previous one
-    // (measured), so a step costs its instruction count; chain_step() is 6.
     uint64_t h = seed;
     int32_t since_key = 0;  // uniform: all lanes step in lockstep from token 0
     lds_barrier();
