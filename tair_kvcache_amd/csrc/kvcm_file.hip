@@ -126,7 +126,7 @@ struct kvcm_file_store {
     std::vector<std::thread> pool;
     int pool_idle = 0;
     bool pool_stop = false;
-    std::atomic<int> reads_in_flight{0};
+    std::atomic<int> transfers_in_flight{0};
 
     void submit(std::function<void()> job) {
         std::lock_guard<std::mutex> lock(pool_mu);
@@ -357,13 +357,13 @@ int32_t move_device_segments(kvcm_file_store *store, int fd, const std::vector<S
     if (e != hipSuccess) {
         return hip_code(e);
     }
-    // Callers that read at the same time share the helper threads: eight callers are eight readers already.
+    // Transfers that run at the same time share the helper threads: eight callers are eight movers already.
     struct InFlight {
         std::atomic<int> &n;
         int now;
         explicit InFlight(std::atomic<int> &counter) : n(counter), now(++counter) {}
         ~InFlight() { --n; }
-    } in_flight(store->reads_in_flight);
+    } in_flight(store->transfers_in_flight);
     const size_t workers =
         put ? 1
             : std::max<size_t>(1, std::min<size_t>(static_cast<size_t>(store->io_threads / in_flight.now),
