@@ -15,8 +15,8 @@ def _keys_with_repeats(rng, n, distinct):
     return base[rng.integers(0, max(distinct, 1), size=n)]
 
 
-@pytest.mark.parametrize("n,distinct", [(1, 1), (2, 1), (63, 5), (64, 64), (1000, 1), (1025, 700), (16384, 12416),
-                                        (65536, 300), (300000, 150000), (1 << 20, 1 << 20)])
+@pytest.mark.parametrize("n,distinct", [(1, 1), (2, 1), (63, 5), (64, 64), (1000, 1), (1025, 700), (8192, 8192), (16383, 16383),
+                                        (16384, 12416), (16384, 16384), (16385, 9000), (65536, 300), (300000, 150000), (1 << 20, 1 << 20)])
 def test_first_occurrence_matches_oracle(oracle, n, distinct):
     from tair_kvcache_amd import save_selection
     rng = np.random.default_rng(n * 7 + distinct)
@@ -41,7 +41,7 @@ def test_first_occurrence_sequential_and_clustered_keys(oracle):
         assert (first.cpu().numpy() == oracle.first_occurrence(keys)[0]).all()
 
 
-@pytest.mark.parametrize("n", [0, 1, 63, 64, 1023, 1024, 1025, 4096, 100000, (1 << 20) + 3, 3 << 20])
+@pytest.mark.parametrize("n", [0, 1, 63, 64, 1023, 1024, 1025, 4096, 16384, 65535, 65536, 65537, 100000, (1 << 20) + 3, 3 << 20])
 @pytest.mark.parametrize("density", [0.0, 0.3, 1.0])
 def test_mask_to_indices_matches_oracle(oracle, n, density):
     from tair_kvcache_amd import save_selection
