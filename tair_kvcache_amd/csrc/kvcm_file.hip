@@ -251,7 +251,7 @@ int32_t plan_segments(const kvcm_file_store *store, const uint64_t *blkids, cons
         uint64_t offset = blkids[b] * bsz;
         for (int32_t k = 0; k < iov_counts[b]; k++) {
             const kvcm_iov &iov = iovs[first + k];
-            if (offset + iov.size > limit) {
+            if (offset > limit || iov.size > limit - offset) {  // written so that a huge size cannot wrap around
                 return KVCM_ERR_INVALID_ARG;
             }
             if (!iov.ignore && iov.base && iov.size > 0) {

@@ -173,6 +173,10 @@ def test_refusals_match_the_oracle(oracle, tmp_path):
     # the URI's size must be the store's block size
     assert oracle.file_put(theirs, bsz, [(0, [ok])], sizes=[255]) == -1
     assert oracle.file_get(theirs, bsz, [(0, [dst])], sizes=[255]) == -1
+    # a size that would wrap the offset arithmetic is refused like any other that reaches beyond the file
+    huge = ct.Iov(type=ct.MemoryType.CPU, base=ok.ctypes.data, size=2**64 - 8, ignore=False)
+    assert sdk.Put([_uri(ours, 0, bsz)], [ct.BlockBuffer(iovs=[_iov(ok[:16]), huge])])[0] == EC.ER_SDKWRITE_ERROR
+    assert sdk.Get([_uri(ours, 0, bsz)], [ct.BlockBuffer(iovs=[_iov(dst[:16]), huge])]) == EC.ER_SDKREAD_ERROR
     # a put never shrinks a file
     assert sdk.Put([_uri(ours, 1, bsz)], [ct.BlockBuffer(iovs=[_iov(ok)])])[0] == EC.ER_OK
     assert os.path.getsize(ours) == 4 * bsz
