@@ -93,3 +93,17 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(_lib.KvcmLibraryError):
         _lib.lib()
+
+
+def test_header_is_plain_c(tmp_path):
+    """A cgo / FFI binding includes the header from C: it must compile as C99 with warnings on, without HIP headers."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "kvcm_hip.h"\n'
+                   "int main(void) { kvcm_iov v; v.type = KVCM_MEMORY_GPU; v.ignore = 0; v.base = 0; v.size = 0;\n"
+                   "  return (int)v.size + (KVCM_ERR_IO == -4 ? 0 : 1); }\n")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+                    "-c", str(src), "-o", str(tmp_path / "use_header.o")], check=True)
