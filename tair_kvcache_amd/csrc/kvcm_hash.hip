@@ -268,16 +268,33 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t r = static_cast<int64_t>(blockIdx.x) * kReqs + lane;
 
-    int64_t my_ntok = 0;
+    // Everything that has to come from memory before the first tile can be requested is asked for here, by all four
+    // waves at once: one trip to memory instead of three in a row (a 64 x 4096 batch is only ~50 us long).
+    int64_t my_ntok = 0, key_pos = 0;
+    LoaderCtx<TokT> ctx;
+    bool buffer_loads = false;
     if (wave == 0) {
         int64_t start = token_offsets[static_cast<int64_t>(blockIdx.x) * kReqs];  // rows past R idle at the first row
         if (r < R) {
             start = token_offsets[r];
             const int64_t n = token_offsets[r + 1] - start;
             my_ntok = (n / block_size) * block_size;  // a trailing partial block yields no key
+            key_pos = key_offsets ? key_offsets[r] : r * ((token_offsets[1] - token_offsets[0]) / block_size);
         }
         s_start[lane] = start;
         s_ntok[lane] = my_ntok;
+    } else {
+        ctx.tokens = tokens;
+        ctx.s_start = s_start;
+        const int64_t total = token_offsets[R];
+        ctx.last_token = total - 1;  // >= 0 whenever a tile is loaded: some request has a full block then
+        const int64_t r_first = static_cast<int64_t>(blockIdx.x) * kReqs;
+        const int64_t r_end = r_first + kReqs < R ? r_first + kReqs : R;
+        ctx.wg_first_token = token_offsets[r_first];
+        const uint64_t to_end = static_cast<uint64_t>(total - ctx.wg_first_token) * sizeof(TokT);
+        ctx.wg_bytes = to_end > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(to_end);
+        const uint64_t wg_span = static_cast<uint64_t>(token_offsets[r_end] - ctx.wg_first_token) * sizeof(TokT);
+        buffer_loads = !force_global_loads && wg_span < 0xFFF00000ull;
     }
     __syncthreads();
 
@@ -303,18 +320,7 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
 
     if (wave != 0) {
         // ---------------------------------------------------------------- loader waves
-        LoaderCtx<TokT> ctx;
-        ctx.tokens = tokens;
-        ctx.s_start = s_start;
-        const int64_t total = token_offsets[R];
-        ctx.last_token = total - 1;  // >= 0 here: some request has a full block
-        const int64_t r_first = static_cast<int64_t>(blockIdx.x) * kReqs;
-        const int64_t r_end = r_first + kReqs < R ? r_first + kReqs : R;
-        ctx.wg_first_token = token_offsets[r_first];
-        const uint64_t to_end = static_cast<uint64_t>(total - ctx.wg_first_token) * sizeof(TokT);
-        ctx.wg_bytes = to_end > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(to_end);
-        const uint64_t wg_span = static_cast<uint64_t>(token_offsets[r_end] - ctx.wg_first_token) * sizeof(TokT);
-        if (!force_global_loads && wg_span < 0xFFF00000ull) {
+        if (buffer_loads) {
             run_loader<BufferLoader<TokT>, TokT>(ctx, s_tile, wave - 1, ntiles, lane);
         } else {
             run_loader<GlobalLoader<TokT>, TokT>(ctx, s_tile, wave - 1, ntiles, lane);
@@ -332,33 +338,42 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         // usable when R is not a multiple of 64.
         return;
     }
-    int64_t key_pos = key_offsets ? key_offsets[r] : r * ((token_offsets[1] - token_offsets[0]) / block_size);
     ulonglong2 cur[kTT / 2], nxt[kTT / 2];
     read_row(cur, &s_tile[0][lane][0]);
+    // Loop control in 32-bit scalars (there are no ordered 64-bit scalar compares, and every vector compare is an issue
+    // slot of this wave): tiles [0, n_full) are those in which no lane has run out of tokens. A request of 2^37 tokens
+    // does not fit the memory of the device, so the tile count fits 32 bits.
+    const int32_t nt = static_cast<int32_t>(ntiles);
+    const int64_t full = min_ntok / kTT;
+    const int32_t n_full = static_cast<int32_t>(full < ntiles ? full : ntiles);
     int ring = 0;
-    for (int64_t k = 0; k < ntiles; k += 2) {
+    for (int32_t k = 0; k < nt; k += 2) {
         // even tile: compute on `cur`, prefetch the odd tile into `nxt`; then the other way round
         int ring1 = ring + 1 == kRing ? 0 : ring + 1;
-        if (k + 1 < ntiles) {
+        if (k + 1 < nt) {
             read_row(nxt, &s_tile[ring1][lane][0]);
         }
-        if ((k + 1) * kTT <= min_ntok) {
-            run_tile<CHUNK, false, BS>(cur, h, k * kTT, my_ntok, since_key, block_size, keys, key_pos);
+        if (k < n_full) {
+            run_tile<CHUNK, false, BS>(cur, h, static_cast<int64_t>(k) * kTT, my_ntok, since_key, block_size, keys,
+                                       key_pos);
         } else {
-            run_tile<CHUNK, true, BS>(cur, h, k * kTT, my_ntok, since_key, block_size, keys, key_pos);
+            run_tile<CHUNK, true, BS>(cur, h, static_cast<int64_t>(k) * kTT, my_ntok, since_key, block_size, keys,
+                                      key_pos);
         }
         lds_barrier();
-        if (k + 1 >= ntiles) {
+        if (k + 1 >= nt) {
             break;
         }
         ring = ring1 + 1 == kRing ? 0 : ring1 + 1;
-        if (k + 2 < ntiles) {
+        if (k + 2 < nt) {
             read_row(cur, &s_tile[ring][lane][0]);
         }
-        if ((k + 2) * kTT <= min_ntok) {
-            run_tile<CHUNK, false, BS>(nxt, h, (k + 1) * kTT, my_ntok, since_key, block_size, keys, key_pos);
+        if (k + 1 < n_full) {
+            run_tile<CHUNK, false, BS>(nxt, h, static_cast<int64_t>(k + 1) * kTT, my_ntok, since_key, block_size, keys,
+                                       key_pos);
         } else {
-            run_tile<CHUNK, true, BS>(nxt, h, (k + 1) * kTT, my_ntok, since_key, block_size, keys, key_pos);
+            run_tile<CHUNK, true, BS>(nxt, h, static_cast<int64_t>(k + 1) * kTT, my_ntok, since_key, block_size, keys,
+                                      key_pos);
         }
         lds_barrier();
     }
