@@ -203,8 +203,10 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
 }
 
 // The chain wave's work on one tile: kTT steps from the lane's pre-added terms `a`, a key at every block
-// boundary. MASKED = some lane may have run out of tokens inside this tile (ragged batch); the common case of
-// equally long requests takes the unmasked path, which has no per-lane compare in it.
+// boundary. MASKED = some lane may have run out of tokens inside this tile (ragged batch). Such a lane keeps stepping
+// -- on a neighbour's tokens or on zeros, whatever the loaders fetched past its end -- because masking the steps would
+// cost the wave a compare, two exec writes and a branch per chunk; its state is dead from there on, and only its KEY
+// STORES are masked. The common case of equally long requests takes the unmasked path, which has no per-lane compare.
 // BS > 0 = the block size is this compile-time constant (a divisor or a multiple of the tile): the places where a key
 // is due are then known when the code is written, and the scalar bookkeeping (add, compare, branch per chunk: one
 // instruction slot in sixteen of the wave that sets the pace) disappears from the loop.
@@ -213,14 +215,15 @@ __device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_
                                          int32_t &since_key, int32_t block_size, int64_t *__restrict__ keys,
                                          int64_t &key_pos) {
     static_assert(BS == 0 || (BS % CHUNK == 0 && (kTT % BS == 0 || BS % kTT == 0)), "block size fits the tiling");
+    // tokens of this lane that are hashed and lie in this tile or before its end: a block that ends at position p of
+    // the tile belongs to the lane iff p <= left (my_ntok is a multiple of the block size)
+    const int64_t left64 = my_ntok - t0;
+    const int32_t left = MASKED ? static_cast<int32_t>(left64 < kTT ? (left64 > 0 ? left64 : 0) : kTT) : kTT;
 #pragma unroll
     for (int c = 0; c < kTT; c += CHUNK) {
-        const bool active = !MASKED || (t0 + c) < my_ntok;
-        if (active) {
 #pragma unroll
-            for (int s = c; s < c + CHUNK; ++s) {
-                h = chain_step(h, (s & 1) ? a[s / 2].y : a[s / 2].x);
-            }
+        for (int s = c; s < c + CHUNK; ++s) {
+            h = chain_step(h, (s & 1) ? a[s / 2].y : a[s / 2].x);
         }
         bool key_due;
         if (BS == 0) {
@@ -235,7 +238,7 @@ __device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_
             key_due = c + CHUNK == kTT && (t0 + kTT) % BS == 0;
         }
         if (key_due) {
-            if (active) {
+            if (!MASKED || c + CHUNK <= left) {
                 keys[key_pos] = static_cast<int64_t>(h);
             }
             key_pos += 1;
