@@ -70,6 +70,15 @@ __device__ __forceinline__ uint64_t chain_step(uint64_t h, uint64_t a) {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+// sign-extended 32-bit token + C in one instruction (the compiler's own form is a shift for the sign and a 64-bit
+// add): with 32-bit tokens the loader wave whose turn it is has twice as many tokens to convert per load, and its
+// store phase must stay shorter than the chain wave's tile
+__device__ __forceinline__ uint64_t pre_add_i32(uint32_t token) {
+    uint64_t sum, carry_out;
+    asm("v_mad_i64_i32 %0, %1, %2, 1, %3" : "=v"(sum), "=s"(carry_out) : "v"(token), "s"(kGolden));
+    return sum;
+}
+
 // What a loader wave needs to know about its workgroup.
 template <typename TokT>
 struct LoaderCtx {
@@ -107,9 +116,14 @@ struct BufferLoader {
         }
     }
     __device__ __forceinline__ void issue(int64_t t0) {
+        issue_half<0>(t0);
+        issue_half<1>(t0);
+    }
+    template <int HALF>
+    __device__ __forceinline__ void issue_half(int64_t t0) {
         const uint32_t tile_off = static_cast<uint32_t>(t0 * sizeof(TokT));
 #pragma unroll
-        for (int j = 0; j < kNL; ++j) {
+        for (int j = HALF * (kNL / 2); j < (HALF + 1) * (kNL / 2); ++j) {
             // aux = 2: the non-temporal bit; tokens are read once (+10 % at 16 384 requests)
             regs[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, rel[j] + tile_off, 0, 2);
         }
@@ -117,6 +131,9 @@ struct BufferLoader {
     // Adds the golden-ratio constant (the token term of the step is v + C) and writes the tile transposed.
     __device__ __forceinline__ void store(uint64_t (*tile)[kTT + kPad]) const {
         const uint32_t sub = lane / kLPR, piece = lane % kLPR;
+        // One wait for all the loads of the tile (they were requested two tile periods ago) instead of one in front
+        // of every LDS write: this phase has to fit into the chain wave's tile, and every instruction of it counts.
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0); lgkmcnt and expcnt left at their maxima
 #pragma unroll
         for (int j = 0; j < kNL; ++j) {
             ulonglong2 *dst = reinterpret_cast<ulonglong2 *>(&tile[j * kRPW + sub][piece * kEPL]);
@@ -125,10 +142,8 @@ struct BufferLoader {
                 dst[0] = make_ulonglong2(((static_cast<uint64_t>(v.y) << 32) | v.x) + kGolden,
                                          ((static_cast<uint64_t>(v.w) << 32) | v.z) + kGolden);
             } else {
-                dst[0] = make_ulonglong2(static_cast<uint64_t>(static_cast<int64_t>(static_cast<int32_t>(v.x))) + kGolden,
-                                         static_cast<uint64_t>(static_cast<int64_t>(static_cast<int32_t>(v.y))) + kGolden);
-                dst[1] = make_ulonglong2(static_cast<uint64_t>(static_cast<int64_t>(static_cast<int32_t>(v.z))) + kGolden,
-                                         static_cast<uint64_t>(static_cast<int64_t>(static_cast<int32_t>(v.w))) + kGolden);
+                dst[0] = make_ulonglong2(pre_add_i32(v.x), pre_add_i32(v.y));
+                dst[1] = make_ulonglong2(pre_add_i32(v.z), pre_add_i32(v.w));
             }
         }
     }
@@ -147,8 +162,13 @@ struct GlobalLoader {
         lane = lane_;
     }
     __device__ __forceinline__ void issue(int64_t t0) {
+        issue_half<0>(t0);
+        issue_half<1>(t0);
+    }
+    template <int HALF>
+    __device__ __forceinline__ void issue_half(int64_t t0) {
 #pragma unroll
-        for (int j = 0; j < kPerLane; ++j) {
+        for (int j = HALF * (kPerLane / 2); j < (HALF + 1) * (kPerLane / 2); ++j) {
             const uint32_t e = lane + 64u * j;
             const int64_t pos = c.s_start[e / kTT] + t0 + (e % kTT);
             regs[j] = c.tokens[pos < c.last_token ? pos : c.last_token];
@@ -187,6 +207,7 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
     }
     int64_t turn = 2 % kLoaders;  // loader whose tile is due: (k + 2) % kLoaders
     int slot = 2;                 // ring slot of that tile: (k + 2) % kRing
+    bool was_mine = false;
     for (int64_t k = 0; k < ntiles; ++k) {
         const int64_t nxt = k + 2;  // tile that must be in LDS when this iteration ends
         const bool mine = turn == lw && nxt < ntiles;
@@ -196,9 +217,15 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
         turn = turn + 1 == kLoaders ? 0 : turn + 1;
         slot = slot + 1 == kRing ? 0 : slot + 1;
         lds_barrier();
+        // the loads of this loader's next tile go out in two halves, one tile period apart: a burst of 32 load
+        // instructions sits in the CU's memory pipeline in front of the chain wave's key stores
         if (mine && nxt + kLoaders < ntiles) {
-            ld.issue((nxt + kLoaders) * kTT);
+            ld.template issue_half<0>((nxt + kLoaders) * kTT);
         }
+        if (was_mine && nxt - 1 + kLoaders < ntiles) {
+            ld.template issue_half<1>((nxt - 1 + kLoaders) * kTT);
+        }
+        was_mine = mine;
     }
 }
 
