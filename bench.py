@@ -28,7 +28,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # HBM bytes per launch of the two copy kernels at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled by a plain 8 GiB copy in the same run (profiles/copy_span_llama3_8b_hbm_traffic.md). Counters cannot be read
 # from inside this process, so the figures are carried here and reported only for the workload they were taken on.
-MEASURED_TRAFFIC = {"unique_blocks": 12416, "gather": 52079227083, "scatter": 52076947905}
+MEASURED_TRAFFIC = {"unique_blocks": 12416, "gather": 52077746636, "scatter": 52079466648}
 
 # Llama-3-8B KV layout: the configuration the headline metric is quoted on
 LAYERS, KV_HEADS, HEAD_DIM, ITEMSIZE = 32, 8, 128, 2
