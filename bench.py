@@ -28,7 +28,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # HBM bytes per launch of the two copy kernels at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled by a plain 8 GiB copy in the same run (profiles/copy_span_llama3_8b_hbm_traffic.md). Counters cannot be read
 # from inside this process, so the figures are carried here and reported only for the workload they were taken on.
-MEASURED_TRAFFIC = {"unique_blocks": 12416, "gather": 52077746636, "scatter": 52079466648}
+MEASURED_TRAFFIC = {"unique_blocks": 12416, "gather": 52077746636, "scatter": 52079466648,
+                    "hash_saturated": int((512.6 + 38.4) * 2**20)}
 
 # Llama-3-8B KV layout: the configuration the headline metric is quoted on
 LAYERS, KV_HEADS, HEAD_DIM, ITEMSIZE = 32, 8, 128, 2
@@ -236,6 +237,7 @@ def main():
     torch.cuda.synchronize()
     ms_sat = e0.elapsed_time(e1) / 3
     sat_keys_per_s = sat_keys.numel() / (ms_sat * 1e-3)
+    sat_alg_bytes = sat_R * TOKENS_PER_REQ * 8 + (sat_R + 1) * 8 * 2 + sat_keys.numel() * 8
     # ... and with four batches of the configuration hashed in one launch (256 chains): the smallest launch that is
     # past 1e9 keys/s, since one batch alone is bound by the latency of its 4096 dependent steps
     few_R = 4 * REQUESTS
@@ -289,6 +291,15 @@ def main():
         "hash_saturated_GBps": round(sat_R * TOKENS_PER_REQ * 8.5 / (ms_sat * 1e-3) / 1e9, 1),
         "verified_against_oracle": verified,
         "roofline": dominant,
+        # the block-key kernel at 16 384 chains: tokens + offsets read, keys written; traffic from the same two
+        # rocprofv3 --pmc runs as the copy kernels (512.6 MiB read + 38.4 MiB written)
+        "roofline_hash_saturated": {"bound": "hbm",
+                                    "achieved": round(sat_alg_bytes / (ms_sat * 1e-3) / 1e9, 1),
+                                    "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                    "frac": round(sat_alg_bytes / (ms_sat * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                                    "traffic": MEASURED_TRAFFIC["hash_saturated"] if sat_R == 16384 else None,
+                                    "kernel": "hash_tokens_kernel<long, 8, 16>", "ms_per_launch": round(ms_sat, 4),
+                                    "algorithmic_bytes_per_launch": sat_alg_bytes},
         "roofline_save": roof_g, "roofline_load": roof_s,
     }
     if not args.no_cpu_baseline:
