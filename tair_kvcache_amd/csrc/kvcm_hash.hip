@@ -124,8 +124,10 @@ struct BufferLoader {
         const uint32_t tile_off = static_cast<uint32_t>(t0 * sizeof(TokT));
 #pragma unroll
         for (int j = HALF * (kNL / 2); j < (HALF + 1) * (kNL / 2); ++j) {
-            // aux = 2: the non-temporal bit; tokens are read once (+10 % at 16 384 requests)
-            regs[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, rel[j] + tile_off, 0, 2);
+            // aux = 2: the non-temporal bit. Tokens are read once; with 8-byte tokens the bit is worth 17 % at
+            // 16 384 requests (107 us against 125 us), with 4-byte tokens it COSTS 10 % (83 us against 75 us),
+            // measured with sc0, sc1 and both as well: only nt matters.
+            regs[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, rel[j] + tile_off, 0, sizeof(TokT) == 8 ? 2 : 0);
         }
     }
     // Adds the golden-ratio constant (the token term of the step is v + C) and writes the tile transposed.
