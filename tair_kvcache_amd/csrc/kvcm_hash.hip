@@ -197,22 +197,25 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
     static_assert(kRing == 3 && kLoaders >= 3, "three ring slots: computed on, prefetched from, written to");
     Loader ld;
     ld.setup(ctx, lane);
-    if (lw < ntiles) {
-        ld.issue(lw * kTT);
+    // 32-bit counters: the loop control stays in scalar registers (there are no ordered 64-bit scalar compares); a
+    // request of 2^37 tokens does not fit the memory of the device
+    const int32_t nt = static_cast<int32_t>(ntiles), me = static_cast<int32_t>(lw);
+    if (me < nt) {
+        ld.issue(static_cast<int64_t>(me) * kTT);
     }
-    if (lw < 2 && lw < ntiles) {
-        ld.store(s_tile[lw]);
+    if (me < 2 && me < nt) {
+        ld.store(s_tile[me]);
     }
     lds_barrier();
-    if (lw < 2 && lw + kLoaders < ntiles) {
-        ld.issue((lw + kLoaders) * kTT);
+    if (me < 2 && me + kLoaders < nt) {
+        ld.issue(static_cast<int64_t>(me + kLoaders) * kTT);
     }
-    int64_t turn = 2 % kLoaders;  // loader whose tile is due: (k + 2) % kLoaders
+    int32_t turn = 2 % kLoaders;  // loader whose tile is due: (k + 2) % kLoaders
     int slot = 2;                 // ring slot of that tile: (k + 2) % kRing
     bool was_mine = false;
-    for (int64_t k = 0; k < ntiles; ++k) {
-        const int64_t nxt = k + 2;  // tile that must be in LDS when this iteration ends
-        const bool mine = turn == lw && nxt < ntiles;
+    for (int32_t k = 0; k < nt; ++k) {
+        const int32_t nxt = k + 2;  // tile that must be in LDS when this iteration ends
+        const bool mine = turn == me && nxt < nt;
         if (mine) {
             ld.store(s_tile[slot]);
         }
@@ -221,11 +224,11 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
         lds_barrier();
         // the loads of this loader's next tile go out in two halves, one tile period apart: a burst of 32 load
         // instructions sits in the CU's memory pipeline in front of the chain wave's key stores
-        if (mine && nxt + kLoaders < ntiles) {
-            ld.template issue_half<0>((nxt + kLoaders) * kTT);
+        if (mine && nxt + kLoaders < nt) {
+            ld.template issue_half<0>(static_cast<int64_t>(nxt + kLoaders) * kTT);
         }
-        if (was_mine && nxt - 1 + kLoaders < ntiles) {
-            ld.template issue_half<1>((nxt - 1 + kLoaders) * kTT);
+        if (was_mine && nxt - 1 + kLoaders < nt) {
+            ld.template issue_half<1>(static_cast<int64_t>(nxt - 1 + kLoaders) * kTT);
         }
         was_mine = mine;
     }
