@@ -84,29 +84,35 @@ def cpu_baseline(np, O, cores):
     ds, keep_s = O.make_desc(pools, staging, run_s, None, B, T, row_bytes, run_tokens=T)
     moved = 2 * B * P * T * row_bytes  # read + write, one direction
 
-    def timed(fn, reps):
-        best = float("inf")
-        for _ in range(reps):
+    cpu_seconds = [0.0]
+
+    def timed(fn, seconds):
+        """Best of as many repetitions as fit into `seconds` (at least two): about 15 s of CPU work over all legs."""
+        best, spent, reps = float("inf"), 0.0, 0
+        while reps < 2 or spent < seconds:
             t0 = time.perf_counter()
             fn()
-            best = min(best, time.perf_counter() - t0)
+            dt = time.perf_counter() - t0
+            best, spent, reps = min(best, dt), spent + dt, reps + 1
+        cpu_seconds[0] += spent
         return best
 
     O.gather_ex(dg, threads=cores)  # warm
-    g1 = timed(lambda: O.gather_ex(dg), 1)
-    s1 = timed(lambda: O.scatter_ex(ds), 1)
-    gn = timed(lambda: O.gather_ex(dg, threads=cores), 3)
-    sn = timed(lambda: O.scatter_ex(ds, threads=cores), 3)
+    g1 = timed(lambda: O.gather_ex(dg), 2.5)
+    s1 = timed(lambda: O.scatter_ex(ds), 2.5)
+    gn = timed(lambda: O.gather_ex(dg, threads=cores), 2.5)
+    sn = timed(lambda: O.scatter_ex(ds, threads=cores), 2.5)
 
     rng = np.random.default_rng(0)
     tok = rng.integers(0, VOCAB, size=(REQUESTS, TOKENS_PER_REQ), dtype=np.int64)
     nkeys = REQUESTS * (TOKENS_PER_REQ // T)
-    h1 = timed(lambda: O.hash_tokens(tok, T), 20)
-    hn = timed(lambda: O.hash_tokens(tok, T, threads=cores), 20)
+    h1 = timed(lambda: O.hash_tokens(tok, T), 1.5)
+    hn = timed(lambda: O.hash_tokens(tok, T, threads=cores), 1.5)
     out = {
         "value": round(2 * moved / (gn + sn) / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
         "sample": (f"save+load of {B} blocks (2 GiB staged) between a 4 GiB host pool at the same layout and host "
-                   f"staging, one memcpy per 32 KiB (layer,K/V,block) chunk, {cores} threads; 64x4096-token hash batch"),
+                   f"staging, one memcpy per 32 KiB (layer,K/V,block) chunk, {cores} threads; 64x4096-token hash batch; "
+                   f"best of the repetitions that fit 2.5 s (copies) or 1.5 s (hash) per leg"),
         "save_GBps_1thr": round(moved / g1 / 1e9, 2), "load_GBps_1thr": round(moved / s1 / 1e9, 2),
         "save_GBps": round(moved / gn / 1e9, 2), "load_GBps": round(moved / sn / 1e9, 2),
         "hash_keys_per_s_1thr": round(nkeys / h1), "hash_keys_per_s": round(nkeys / hn),
@@ -118,8 +124,9 @@ def cpu_baseline(np, O, cores):
         koff = np.arange(REQUESTS + 1, dtype=np.int64) * (TOKENS_PER_REQ // T)
         keys = np.zeros(nkeys, dtype=np.int64)
         hr = timed(lambda: ref.kvcm_refsrc_hash_tokens(flat.ctypes.data, toff.ctypes.data, REQUESTS, T,
-                                                      keys.ctypes.data, koff.ctypes.data), 20)
+                                                      keys.ctypes.data, koff.ctypes.data), 1.5)
         out["hash_keys_per_s_reference_1thr"] = round(nkeys / hr)
+    out["cpu_seconds"] = round(cpu_seconds[0], 1)
     return out
 
 
