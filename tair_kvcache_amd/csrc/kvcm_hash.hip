@@ -564,6 +564,8 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
         KVCM_LAUNCH_HASH(8, 64);
     } else if (block_size == 128) {
         KVCM_LAUNCH_HASH(8, 128);
+    } else if (block_size == 1) {  // the prefix chain over digests: a key after every step
+        KVCM_LAUNCH_HASH(1, 1);
     } else if (block_size % 8 == 0) {
         KVCM_LAUNCH_HASH(8, 0);
     } else {
