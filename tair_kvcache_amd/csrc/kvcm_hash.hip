@@ -287,7 +287,7 @@ __device__ __forceinline__ void read_row(ulonglong2 (&a)[kTT / 2], const uint64_
 }
 
 // CHUNK = steps between two looks at the block boundary: 8 when block_size % 8 == 0 (a lane is then
-// active for whole chunks or not at all), otherwise 1. BS = block size when it is 16, 32, 64 or 128, otherwise 0.
+// active for whole chunks or not at all), otherwise 1. BS = block size when it is 1, 8, 16, 32, 64 or 128, otherwise 0.
 template <typename TokT, int CHUNK, int BS>
 __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__restrict__ tokens,
                                                               const int64_t *__restrict__ token_offsets, int32_t R,
@@ -558,6 +558,8 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
                        d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
     if (block_size == 16) {  // the engines' usual block sizes get kernels of their own
         KVCM_LAUNCH_HASH(8, 16);
+    } else if (block_size == 8) {
+        KVCM_LAUNCH_HASH(8, 8);
     } else if (block_size == 32) {
         KVCM_LAUNCH_HASH(8, 32);
     } else if (block_size == 64) {
