@@ -219,6 +219,21 @@ int32_t kvcm_hip_first_occurrence(const int64_t *d_keys, int64_t n, void *d_work
                                   int32_t *d_first_idx, uint8_t *d_is_repeat, kvcm_stream_t stream);
 
 /*
+ * kvcm_hip_first_occurrence without a workspace argument and without any allocation: the table lives in a device
+ * array that is part of the library's code object (8 MiB per GPU the library is used on, held until the process
+ * ends). No counterpart in the reference. It is for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc. Same results as kvcm_hip_first_occurrence.
+ * n <= kvcm_hip_first_occurrence_static_max_keys() = 2^20, KVCM_ERR_TOO_LARGE beyond. The device that is current at
+ * the call is the one whose table is used; its address is looked up on the first call per device (a call with n = 0
+ * does just that and launches nothing: make it before a capture starts). All calls on one GPU share that GPU's table:
+ * calls that overlap on one GPU (two streams, or two threads) race and give undefined results; serialise them, or use
+ * kvcm_hip_first_occurrence with a workspace per call.
+ */
+int64_t kvcm_hip_first_occurrence_static_max_keys(void);
+int32_t kvcm_hip_first_occurrence_static(const int64_t *d_keys, int64_t n, int32_t *d_first_idx, uint8_t *d_is_repeat,
+                                         kvcm_stream_t stream);
+
+/*
  * Indices of the blocks to save, ascending: every i < n with d_mask[i] == 0 (and d_mask2[i] == 0 when d_mask2 is
  * not NULL) is appended to d_indices (int32, room for n entries); their number goes to *d_count (device int32).
  * Replaces: TairKvCacheConnector.parse_block_mask_to_save_indices, bool_masks branch

@@ -64,6 +64,8 @@ SIGNATURES = {
     "kvcm_hip_generate_blocks_idx": (i32, [vp, i32, vp, i32, i32, i32, vp, vp, vp]),
     "kvcm_hip_first_occurrence_workspace_bytes": (i64, [i64]),
     "kvcm_hip_first_occurrence": (i32, [vp, i64, vp, i64, vp, vp, vp]),
+    "kvcm_hip_first_occurrence_static_max_keys": (i64, []),
+    "kvcm_hip_first_occurrence_static": (i32, [vp, i64, vp, vp, vp]),
     "kvcm_hip_mask_to_indices_workspace_bytes": (i64, [i64]),
     "kvcm_hip_mask_to_indices": (i32, [vp, vp, i64, vp, i64, vp, vp, vp]),
     "kvcm_hip_iov_crc32": (i32, [vp, i32, vp, sz, vp]),

@@ -7,10 +7,56 @@
 // (kvcm_hip_hash_tokens) and to the index kernels that consume the list.
 //
 // Small integer kernels, nowhere near a bandwidth bound: n is the number of block keys of a batch (thousands).
+#include <atomic>
+#include <mutex>
+
 #include "kvcm_internal.h"
 
 namespace kvcm {
 namespace {
+
+// Table of kvcm_hip_first_occurrence_static: room for 2^20 keys (capacity 2 n, one int32 per slot = 8 MiB).
+// Every device that the library runs on holds its own copy, at its own address, until the process ends.
+constexpr int64_t kStaticMaxKeys = int64_t{1} << 20;
+constexpr int64_t kStaticCapacity = 2 * kStaticMaxKeys;
+static __device__ __align__(256) int32_t scratch[kStaticCapacity];
+
+// Device address of `scratch` per device: in host code the array's name is only a handle for the runtime's symbol
+// calls, never an address a kernel may be given.
+constexpr int kMaxDevices = 64;
+std::atomic<int32_t *> g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+// The current device's copy of `scratch`; looked up once per device. Returns a kvcm / HIP code.
+int32_t static_scratch(int32_t **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        return static_cast<int32_t>(e);
+    }
+    if (dev < 0 || dev >= kMaxDevices) {
+        return KVCM_ERR_TOO_LARGE;
+    }
+    int32_t *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        std::lock_guard<std::mutex> guard(g_scratch_mutex);
+        p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+        if (!p) {
+            void *addr = nullptr;
+            e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess) {
+                return static_cast<int32_t>(e);
+            }
+            if (!addr) {
+                return static_cast<int32_t>(hipErrorInvalidSymbol);
+            }
+            p = static_cast<int32_t *>(addr);
+            g_scratch_ptr[dev].store(p, std::memory_order_release);
+        }
+    }
+    *out = p;
+    return KVCM_OK;
+}
 
 constexpr int kSelThreads = 1024;  // 16 waves: one workgroup scans 1024 flags or counts per pass
 constexpr int kSelWaves = kSelThreads / 64;
@@ -157,6 +203,22 @@ int64_t table_capacity(int64_t n) {
     return cap;
 }
 
+// fill / insert / resolve on a table of `cap` slots (a power of two, >= 2 n); the fill is a kernel, so the
+// sequence may be recorded into a graph.
+int32_t launch_first_occurrence(const int64_t *d_keys, int64_t n, int32_t *table, int64_t cap, int32_t *d_first_idx,
+                                uint8_t *d_is_repeat, hipStream_t s) {
+    int log2cap = 0;
+    while ((int64_t{1} << log2cap) < cap) {
+        log2cap++;
+    }
+    const int32_t n32 = static_cast<int32_t>(n);
+    const unsigned groups = static_cast<unsigned>((n + 255) / 256);
+    fill_i32_kernel<<<static_cast<unsigned>(cap / 256), 256, 0, s>>>(table, cap, -1);
+    insert_kernel<<<groups, 256, 0, s>>>(d_keys, n32, table, static_cast<uint32_t>(cap - 1), 64 - log2cap, d_first_idx);
+    resolve_kernel<<<groups, 256, 0, s>>>(d_first_idx, table, n32, d_is_repeat);
+    return launch_status();
+}
+
 }  // namespace
 }  // namespace kvcm
 
@@ -190,19 +252,35 @@ int32_t kvcm_hip_first_occurrence(const int64_t *d_keys, int64_t n, void *d_work
     if (reinterpret_cast<uintptr_t>(d_workspace) % 4 != 0) {
         return KVCM_ERR_ALIGNMENT;
     }
-    int log2cap = 0;
-    while ((int64_t{1} << log2cap) < cap) {
-        log2cap++;
+    return kvcm::launch_first_occurrence(d_keys, n, static_cast<int32_t *>(d_workspace), cap, d_first_idx, d_is_repeat,
+                                         static_cast<hipStream_t>(stream));
+}
+
+int64_t kvcm_hip_first_occurrence_static_max_keys(void) { return kvcm::kStaticMaxKeys; }
+
+int32_t kvcm_hip_first_occurrence_static(const int64_t *d_keys, int64_t n, int32_t *d_first_idx, uint8_t *d_is_repeat,
+                                         kvcm_stream_t stream) {
+    if (n < 0) {
+        return KVCM_ERR_INVALID_ARG;
     }
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    int32_t *table = static_cast<int32_t *>(d_workspace);
-    const int32_t n32 = static_cast<int32_t>(n);
-    const unsigned groups = static_cast<unsigned>((n + 255) / 256);
-    kvcm::fill_i32_kernel<<<static_cast<unsigned>(cap / 256), 256, 0, s>>>(table, cap, -1);
-    kvcm::insert_kernel<<<groups, 256, 0, s>>>(d_keys, n32, table, static_cast<uint32_t>(cap - 1), 64 - log2cap,
-                                                d_first_idx);
-    kvcm::resolve_kernel<<<groups, 256, 0, s>>>(d_first_idx, table, n32, d_is_repeat);
-    return kvcm::launch_status();
+    if (n > kvcm::kStaticMaxKeys) {
+        return KVCM_ERR_TOO_LARGE;
+    }
+    if (n > 0 && (!d_keys || !d_first_idx)) {
+        return KVCM_ERR_INVALID_ARG;
+    }
+    // also for n == 0: a call with no keys is how a caller does the per-device set-up ahead of time
+    int32_t *table = nullptr;
+    const int32_t rc = kvcm::static_scratch(&table);
+    if (rc != KVCM_OK) {
+        return rc;
+    }
+    if (n == 0) {
+        return KVCM_OK;
+    }
+    // the table keeps the last call's contents: the fill kernel clears the slots this call probes
+    return kvcm::launch_first_occurrence(d_keys, n, table, kvcm::table_capacity(n), d_first_idx, d_is_repeat,
+                                         static_cast<hipStream_t>(stream));
 }
 
 int64_t kvcm_hip_mask_to_indices_workspace_bytes(int64_t n) {
