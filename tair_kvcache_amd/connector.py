@@ -2,48 +2,58 @@
 
     generate_blocks_idx   TairKvCacheConnector.generate_blocks_idx  kv_cache_manager/py_connector/vllm/v1_connector.py:308-320
     register_kv_caches    TairKvCacheConnector.register_kv_caches   kv_cache_manager/py_connector/vllm/v1_connector.py:360-445
+    KVCacheInfo           kv_cache_manager/py_connector/common/types.py:9-23
     MultiResult           kv_cache_manager/py_connector/vllm/data_transfer.py:18-36
-    DataTransferManager   kv_cache_manager/py_connector/vllm/data_transfer.py:39-244 (save_task :190-244, load_task :108-158)
+    DataTransferManager   kv_cache_manager/py_connector/vllm/data_transfer.py:39-278 (constructor :47-78, load_task
+                          :108-158, create_load_done_callback :160-188, save_task :190-244,
+                          create_save_done_callback :246-278)
 
 What is not here: the engine plugin classes, the HTTP manager client and the ZMQ coordinator (control plane).
 The transfer client is whatever object offers SaveKvCaches(uris, buffers) -> (code, uris) and
-LoadKvCaches(uris, buffers) -> code (kv_cache_manager/client/include/transfer_client.h:19-21).
+LoadKvCaches(uris, buffers) -> code (kv_cache_manager/client/include/transfer_client.h:19-21); the coordinator client
+is whatever object offers send(bytes) (TpCoordinatorClient, kv_cache_manager/py_connector/common/tp_coordinator.py).
 """
 import math
 import threading
+import time
 from concurrent.futures import ThreadPoolExecutor
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, List, Optional, Sequence
+from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
 
 import torch
 
-from . import _lib, client_types
+from . import _lib, client_types, coordinator_messages
 from ._torch_util import as_device_i32, lib, ptr, stream_handle
 from .kernel import batch_gather_scatter_helper
 from .kernel.gather_scatter_helper import CopyBufferAllocator
 
 
 def generate_blocks_idx(manager_block_idxes: Sequence[int], local_block_ids: Sequence[int],
-                        manager_block_size: int, local_block_size: int, device="cuda") -> torch.Tensor:
+                        manager_block_size: int, local_block_size: int, device="cuda",
+                        error_flag: Optional[torch.Tensor] = None) -> torch.Tensor:
     """int32 device tensor [B, manager_block_size]:
     out[b][i] = local_block_ids[tok // local_block_size] * local_block_size + tok % local_block_size with
     tok = manager_block_idxes[b] * manager_block_size + i. The reference builds this as nested Python lists;
-    here it is one kernel and the result never visits the host. Raises AssertionError, as the reference's
-    assert does, when a manager block reaches beyond local_block_ids."""
+    here it is one kernel and the result never visits the host.
+
+    A manager block that reaches beyond local_block_ids: with Python sequences this raises AssertionError before
+    anything is launched, as the reference's assert does. With tensor arguments nothing is read back (no
+    synchronisation): the kernel writes -1 for such entries, which the gather/scatter kernels skip, and raises
+    `error_flag` (an int32 device tensor of one element, if given) to 1."""
     T_mgr, T_eng = int(manager_block_size), int(local_block_size)
     B = len(manager_block_idxes)
     out = torch.empty((B, T_mgr), dtype=torch.int32, device=device)
     if B == 0:
         return out
-    hi = max(manager_block_idxes) if not isinstance(manager_block_idxes, torch.Tensor) else int(
-        manager_block_idxes.max().item())
-    lo = min(manager_block_idxes) if not isinstance(manager_block_idxes, torch.Tensor) else int(
-        manager_block_idxes.min().item())
-    if lo < 0 or (hi * T_mgr + T_mgr - 1) // T_eng >= len(local_block_ids):
-        raise AssertionError("manager block reaches beyond local_block_ids")
+    if not isinstance(manager_block_idxes, torch.Tensor):
+        lo, hi = min(manager_block_idxes), max(manager_block_idxes)
+        if lo < 0 or (hi * T_mgr + T_mgr - 1) // T_eng >= len(local_block_ids):
+            raise AssertionError("manager block reaches beyond local_block_ids")
+    if error_flag is not None and (not error_flag.is_cuda or error_flag.dtype != torch.int32 or error_flag.numel() < 1):
+        raise ValueError("error_flag must be an int32 tensor on the GPU")
     m = as_device_i32(manager_block_idxes, out.device, "manager_block_idxes")
     l = as_device_i32(local_block_ids, out.device, "local_block_ids")
-    rc = lib().kvcm_hip_generate_blocks_idx(ptr(m), B, ptr(l), l.numel(), T_mgr, T_eng, ptr(out), None,
+    rc = lib().kvcm_hip_generate_blocks_idx(ptr(m), B, ptr(l), l.numel(), T_mgr, T_eng, ptr(out), ptr(error_flag),
                                             stream_handle(out.device))
     _lib.check(rc, "kvcm_hip_generate_blocks_idx")
     return out
@@ -60,26 +70,28 @@ def generate_run_starts(manager_block_idxes: Sequence[int], local_block_ids: Seq
     return groups * g, g
 
 
-@dataclass
+@dataclass(frozen=True)
 class KVCacheInfo:
-    """What register_kv_caches derives from the engine's cache tensors (kv_cache_manager/py_connector/common/types.py)."""
+    """What register_kv_caches derives from the engine's cache tensors: the reference's value class, same field names
+    and positional order (kv_cache_manager/py_connector/common/types.py:9-23; built positionally at
+    kv_cache_manager/py_connector/vllm/v1_connector.py:416-430)."""
     tp_rank: int
-    tp_size: int
-    kv_caches: Dict[str, torch.Tensor]
+    world_size: int
+    kvcaches: Dict[str, torch.Tensor]
     kvcache_ptr_tensor_cpu: torch.Tensor
     kvcache_ptr_tensor_gpu: torch.Tensor
     all_kvcache_ptr_tensor_gpu: torch.Tensor
     layer_num: int
     local_token_num: int
-    per_manager_location_spec_shape: tuple
-    per_manager_location_spec_byte_size: int
+    per_manager_block_shape: Tuple[int, ...]
+    per_manager_block_byte_size: int
     per_token_per_layer_dim_size: int
     device: torch.device
     dtype: torch.dtype
 
 
 def register_kv_caches(kv_caches: Dict[str, torch.Tensor], manager_block_size: int, local_block_size: int,
-                       use_mla: bool = False, tp_rank: int = 0, tp_size: int = 1) -> KVCacheInfo:
+                       use_mla: bool = False, tp_rank: int = 0, world_size: int = 1) -> KVCacheInfo:
     """Pointer tables and staging geometry for per-layer caches [2, block_num, block_size, kv_heads, head_dim]
     (MLA: [block_num, block_size, latent_dim], one pointer per layer).
 
@@ -113,7 +125,7 @@ def register_kv_caches(kv_caches: Dict[str, torch.Tensor], manager_block_size: i
             all_ptrs.append(kv_caches[n][0].data_ptr())
             all_ptrs.append(kv_caches[n][1].data_ptr())
     device = first.device
-    return KVCacheInfo(tp_rank, tp_size, kv_caches, ptr_cpu, ptr_cpu.to(device),
+    return KVCacheInfo(tp_rank, world_size, kv_caches, ptr_cpu, ptr_cpu.to(device),
                        torch.tensor(all_ptrs, dtype=torch.int64).to(device), len(kv_caches),
                        block_num * local_block_size, tuple(spec_shape), spec_bytes, dim, device, first.dtype)
 
@@ -153,12 +165,22 @@ class DataTransferManager:
 
     def __init__(self, kvcache_info: KVCacheInfo, manager_block_size: int,
                  copy_buffer_allocator: CopyBufferAllocator, transfer_client: Any,
-                 client_module: Any = client_types, max_workers: int = 32):
+                 coordinator_client: Any = None, extra_config: Any = None, *,
+                 client_module: Any = client_types, message_module: Any = coordinator_messages,
+                 max_workers: int = 32):
+        """The six positional arguments are the reference's (data_transfer.py:47-53; call site
+        kv_cache_manager/py_connector/vllm/v1_connector.py:435-442). Keyword-only extras: `client_module` supplies
+        Iov / BlockBuffer / MemoryType / ClientErrorCode (the pybind module kvcm_py_client, or the plain-Python twin),
+        `message_module` the coordinator message classes and their serialiser, `max_workers` the size of the I/O
+        thread pool (32 in the reference, :89-93)."""
         self._kvcache_info = kvcache_info
         self._manager_block_size = manager_block_size
         self._copy_buffer_allocator = copy_buffer_allocator
         self._transfer_client = transfer_client
+        self._coordinator_client = coordinator_client
+        self._extra_config = extra_config
         self._cm = client_module
+        self._mm = message_module
         device = kvcache_info.device
 
         def init_worker():
@@ -166,9 +188,29 @@ class DataTransferManager:
 
         self._io_executor = ThreadPoolExecutor(max_workers=max_workers, thread_name_prefix="kvcm_io_",
                                                initializer=init_worker)
-        with torch.cuda.device(device):
-            self._save_stream = torch.cuda.Stream()
-            self._load_stream = torch.cuda.Stream()
+        # one save and one load stream (data_transfer.py:77-78), made when the first task needs them so that the
+        # object, its callbacks and its result plumbing can be built and tested where there is no GPU
+        self._stream_lock = threading.Lock()
+        self._streams: Dict[str, Any] = {}
+
+    def _stream(self, which: str):
+        s = self._streams.get(which)
+        if s is None:
+            with self._stream_lock:
+                s = self._streams.get(which)
+                if s is None:
+                    with torch.cuda.device(self._kvcache_info.device):
+                        s = torch.cuda.Stream()
+                    self._streams[which] = s
+        return s
+
+    @property
+    def _save_stream(self):
+        return self._stream("save")
+
+    @property
+    def _load_stream(self):
+        return self._stream("load")
 
     def submit_task(self, func, *args, **kwargs):
         return self._io_executor.submit(func, *args, **kwargs)
@@ -216,6 +258,44 @@ class DataTransferManager:
         finally:
             self._copy_buffer_allocator.free_buffer(slots)
         multi_result.submit_result(task_idx, [result] * len(remote_uris))
+
+    def create_load_done_callback(self, req_id, tp_rank, epoch, local_block_ids):
+        """Callback for a MultiResult of load tasks (data_transfer.py:160-188): walks the per-block result codes of all
+        tasks in order, collects local_block_ids[i] for every block i whose code is not ER_OK, and sends a
+        LoadBlockFinishedEvent with that list to the coordinator."""
+        ok = self._cm.ClientErrorCode.ER_OK
+
+        def generate_message(task_results):
+            failed_block_idxs = []
+            idx = 0
+            for task_result in task_results:
+                for block_result in task_result:
+                    if block_result != ok:
+                        failed_block_idxs.append(local_block_ids[idx])
+                    idx += 1
+            event = self._mm.LoadBlockFinishedEvent(request_id=req_id, tp_rank=tp_rank, epoch=epoch,
+                                                    failed_block_idxs=failed_block_idxs)
+            self._send(self._mm.CoordinateMessage(time.time(), event))
+
+        return generate_message
+
+    def create_save_done_callback(self, req_id, tp_rank, write_session_id):
+        """Callback for a MultiResult of save tasks (data_transfer.py:246-278): one success flag per block, in task
+        order, sent to the coordinator as a SendBlockFinishedEvent."""
+        ok = self._cm.ClientErrorCode.ER_OK
+
+        def generate_message(task_results):
+            is_successes = [block_result == ok for task_result in task_results for block_result in task_result]
+            event = self._mm.SendBlockFinishedEvent(request_id=req_id, tp_rank=tp_rank,
+                                                    write_session_id=write_session_id, is_success_list=is_successes)
+            self._send(self._mm.CoordinateMessage(time.time(), event))
+
+        return generate_message
+
+    def _send(self, message):
+        if self._coordinator_client is None:
+            raise RuntimeError("DataTransferManager was built without a coordinator client: nothing to send to")
+        self._coordinator_client.send(self._mm.CoordinateMsgSerializer.dumps(message))
 
     def save_task(self, multi_result: MultiResult, task_idx: int, remote_uris: List[str], block_token_indices,
                   kvcache_ready_event: Optional[torch.cuda.Event] = None):

@@ -219,7 +219,7 @@ def test_save_to_files_then_load_through_the_transfer_manager(oracle, tmp_path):
     np_caches = [rng.integers(0, 65536, size=(2, nblk, T_eng, H, hd), dtype=np.uint16) for _ in range(L)]
     kv = {f"layer{l}": dev(np_caches[l]).view(torch.float16) for l in range(L)}
     info = connector.register_kv_caches(kv, manager_block_size=T_mgr, local_block_size=T_eng)
-    alloc = CopyBufferAllocator(torch.device("cuda"), torch.float16, list(info.per_manager_location_spec_shape), 16)
+    alloc = CopyBufferAllocator(torch.device("cuda"), torch.float16, list(info.per_manager_block_shape), 16)
     bsz = alloc.slot_nbytes
     client = LocalFileTransferClient(bsz, bounce_bytes=32 * 1024)
     mgr = connector.DataTransferManager(info, T_mgr, alloc, client, max_workers=2)

@@ -86,11 +86,11 @@ def test_save_then_load_through_the_transfer_manager(oracle):
     np_caches = [rng.integers(0, 65536, size=(2, nblk, T, H, hd), dtype=np.uint16) for _ in range(L)]
     kv = {f"layer{l}": dev(np_caches[l]).view(torch.bfloat16) for l in range(L)}
     info = connector.register_kv_caches(kv, manager_block_size=T, local_block_size=T)
-    assert info.per_manager_location_spec_shape == (L, 2, T, H * hd)
-    assert info.per_manager_location_spec_byte_size == L * 2 * T * H * hd * 2
+    assert info.per_manager_block_shape == (L, 2, T, H * hd)
+    assert info.per_manager_block_byte_size == L * 2 * T * H * hd * 2
     assert info.all_kvcache_ptr_tensor_gpu.tolist() == [x for l in range(L) for x in
                                                         (kv[f"layer{l}"][0].data_ptr(), kv[f"layer{l}"][1].data_ptr())]
-    alloc = CopyBufferAllocator(torch.device("cpu"), torch.bfloat16, list(info.per_manager_location_spec_shape), 32)
+    alloc = CopyBufferAllocator(torch.device("cpu"), torch.bfloat16, list(info.per_manager_block_shape), 32)
     client = FakeTransferClient()
     mgr = connector.DataTransferManager(info, T, alloc, client, max_workers=4)
     local_block_ids = cases.block_table(nblk, 24).tolist()
@@ -103,7 +103,7 @@ def test_save_then_load_through_the_transfer_manager(oracle):
     multi = connector.MultiResult(2, lambda r: (results.append(r), done.set()))
     ready = torch.cuda.Event()
     ready.record()
-    uris = [f"file:///kv/blk?blkid={i}&size={info.per_manager_location_spec_byte_size}" for i in range(24)]
+    uris = [f"file:///kv/blk?blkid={i}&size={info.per_manager_block_byte_size}" for i in range(24)]
     mgr.submit_task(mgr.save_task, multi, 0, uris[:12], idx_h[:12].tolist(), ready)
     mgr.submit_task(mgr.save_task, multi, 1, uris[12:], idx[12:], ready)
     assert done.wait(60)
@@ -153,6 +153,128 @@ def test_save_then_load_through_the_transfer_manager(oracle):
     assert res4[0] == [[ClientErrorCode.ER_SDKWRITE_ERROR] * 3] and alloc._inuse_count == 0
     for m in (mgr, mgr2, mgr3, mgr4):
         m.shutdown()
+
+
+class FakeCoordinatorClient:
+    """Stands in for TpCoordinatorClient: records the messages and says when one has arrived."""
+
+    def __init__(self):
+        self.sent = []
+        self.arrived = threading.Event()
+
+    def send(self, data):
+        self.sent.append(data)
+        self.arrived.set()
+
+    def take(self):
+        assert self.arrived.wait(60)
+        self.arrived.clear()
+        return self.sent.pop()
+
+
+def test_worker_loops_of_the_connector_run_on_the_manager_unchanged(oracle):
+    """wait_for_save and start_load_kv as the reference writes them (v1_connector.py:448-475,486-519): the manager is
+    built with the six positional arguments, tasks of block_per_*_task blocks go to the thread pool, the done
+    callbacks fold the per-block codes into the message for the coordinator. One load task is made to fail: its local
+    block ids come back in failed_block_idxs and its blocks stay untouched."""
+    import copy
+    import math
+    from tair_kvcache_amd import connector, coordinator_messages as cm
+    from tair_kvcache_amd.client_types import ClientErrorCode
+    from tair_kvcache_amd.kernel.gather_scatter_helper import CopyBufferAllocator
+
+    class ExtraConfig:
+        block_per_save_task = 8
+        block_per_load_task = 6
+
+    L, nblk, T, H, hd = 3, 64, 16, 2, 64
+    rng = np.random.default_rng(3)
+    np_caches = [rng.integers(0, 65536, size=(2, nblk, T, H, hd), dtype=np.uint16) for _ in range(L)]
+    kv = {f"layer{l}": dev(np_caches[l]).view(torch.bfloat16) for l in range(L)}
+    info = connector.register_kv_caches(kv, T, T, tp_rank=0, world_size=1)
+    alloc = CopyBufferAllocator(torch.device("cuda"), torch.bfloat16, list(info.per_manager_block_shape), 16)
+    client, coord, extra = FakeTransferClient(), FakeCoordinatorClient(), ExtraConfig()
+
+    # the staging pool is in HBM: this fake client finds the slot tensor behind an iov's address
+    def slot_of(iov):
+        raw = alloc._raw_buffer
+        k, rem = divmod(iov.base - raw.data_ptr(), raw[0].numel() * raw.element_size())
+        assert rem == 0 and iov.size == raw[0].numel() * raw.element_size()
+        return raw[k]
+
+    def save(uris, buffers):
+        for uri, buf in zip(uris, buffers):
+            client.store[uri] = slot_of(buf.iovs[0]).view(torch.int16).cpu().numpy().tobytes()
+        return (ClientErrorCode.ER_OK, list(uris))
+
+    def load(uris, buffers):
+        if any("blkid=7&" in u for u in uris):
+            return ClientErrorCode.ER_SDKREAD_ERROR
+        for uri, buf in zip(uris, buffers):
+            slot = slot_of(buf.iovs[0])
+            data = torch.frombuffer(bytearray(client.store[uri]), dtype=torch.int16).view(slot.shape)
+            slot.view(torch.int16).copy_(data)
+        return ClientErrorCode.ER_OK
+
+    client.SaveKvCaches, client.LoadKvCaches = save, load
+    data_transfer = connector.DataTransferManager(info, T, alloc, client, coord, extra)
+
+    local_block_ids = cases.block_table(nblk, 20).tolist()
+    manager_block_idxes = list(range(20))
+    all_remote_uris = [f"file:///kv/f?blkid={i}&size={info.per_manager_block_byte_size}" for i in range(20)]
+
+    # ---- wait_for_save ----
+    kvcache_ready_event = torch.cuda.Event()
+    kvcache_ready_event.record(torch.cuda.current_stream())
+    blocks_idx = connector.generate_blocks_idx(manager_block_idxes, local_block_ids, T, T)
+    per_task_size = extra.block_per_save_task
+    task_num = math.ceil(len(blocks_idx) / per_task_size)
+    done_callback = data_transfer.create_save_done_callback("req-1", info.tp_rank, "session-1")
+    multi_result = connector.MultiResult(task_num, done_callback)
+    task_idx = 0
+    for i in range(0, len(blocks_idx), per_task_size):
+        end_idx = min(len(blocks_idx), i + per_task_size)
+        data_transfer.submit_task(data_transfer.save_task, multi_result, task_idx, all_remote_uris[i:end_idx],
+                                  blocks_idx[i:end_idx], kvcache_ready_event)
+        task_idx += 1
+    msg = cm.CoordinateMsgSerializer.loads(coord.take())
+    assert isinstance(msg.content, cm.SendBlockFinishedEvent) and msg.content.is_success_list == [True] * 20
+    assert (msg.content.request_id, msg.content.write_session_id) == ("req-1", "session-1")
+    idx_h = host(blocks_idx, np.int32)
+    pools = [np_caches[l][kvi].reshape(nblk * T, H * hd) for l in range(L) for kvi in (0, 1)]
+    want = np.zeros((20, 2 * L, T, H * hd), dtype=np.uint16)
+    oracle.batch_gather(pools, want, idx_h, None, T, H * hd * 2)
+    for i, uri in enumerate(all_remote_uris):
+        assert client.store[uri] == want[i].tobytes()
+
+    # ---- start_load_kv into an empty cache; the task that holds block 7 fails ----
+    kv2 = {k: torch.zeros_like(v) for k, v in kv.items()}
+    info2 = connector.register_kv_caches(kv2, T, T)
+    data_transfer2 = connector.DataTransferManager(info2, T, alloc, client, coord, extra)
+    block_token_indices = idx_h.tolist()   # the reference's nested Python lists
+    per_task_size = extra.block_per_load_task
+    task_num = math.ceil(len(block_token_indices) / per_task_size)
+    done_callback = data_transfer2.create_load_done_callback("req-1", info2.tp_rank, 5, copy.copy(local_block_ids))
+    multi_result = connector.MultiResult(task_num, done_callback)
+    task_idx = 0
+    for i in range(0, len(block_token_indices), per_task_size):
+        end_idx = min(len(block_token_indices), i + per_task_size)
+        data_transfer2.submit_task(data_transfer2.load_task, multi_result, task_idx, all_remote_uris[i:end_idx],
+                                   block_token_indices[i:end_idx])
+        task_idx += 1
+    msg = cm.CoordinateMsgSerializer.loads(coord.take())
+    assert isinstance(msg.content, cm.LoadBlockFinishedEvent) and msg.content.epoch == 5
+    assert msg.content.failed_block_idxs == local_block_ids[6:12]   # the second task of six blocks
+    sync()
+    assert alloc._inuse_count == 0
+    loaded = np.array(local_block_ids[:6] + local_block_ids[12:])
+    rest = np.setdiff1d(np.arange(nblk), loaded)
+    for l in range(L):
+        g = host(kv2[f"layer{l}"].view(torch.int16), np.uint16)
+        assert (g[:, loaded] == np_caches[l][:, loaded]).all()
+        assert not g[:, rest].any()
+    data_transfer.shutdown()
+    data_transfer2.shutdown()
 
 
 def test_entry_points_can_be_captured_in_a_hip_graph(oracle):
@@ -297,7 +419,7 @@ def test_transfer_manager_with_staging_in_hbm(oracle):
     np_caches = [rng.integers(0, 65536, size=(2, nblk, T_eng, H, hd), dtype=np.uint16) for _ in range(L)]
     kv = {f"layer{l}": dev(np_caches[l]).view(torch.float16) for l in range(L)}
     info = connector.register_kv_caches(kv, manager_block_size=T_mgr, local_block_size=T_eng)
-    alloc = CopyBufferAllocator(torch.device("cuda"), torch.float16, list(info.per_manager_location_spec_shape), 16)
+    alloc = CopyBufferAllocator(torch.device("cuda"), torch.float16, list(info.per_manager_block_shape), 16)
     client = DeviceStagingClient(alloc)
     mgr = connector.DataTransferManager(info, T_mgr, alloc, client, max_workers=2)
     local_block_ids = cases.block_table(nblk, 24).tolist()  # 24 engine blocks = 12 manager blocks of 32 tokens

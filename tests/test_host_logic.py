@@ -1,4 +1,5 @@
 """Host-side mirror of the reference's Python interface: staging-slot pool, result fan-in, argument checks (no GPU)."""
+import inspect
 import threading
 import time
 
@@ -135,16 +136,16 @@ def test_register_kv_caches_pointer_order_and_spec_size():
     # v1_connector.py:360-445: layer-major, K before V; slot shape [layers, 2, manager_block, heads*dim]
     from tair_kvcache_amd import connector
     kv = _vllm_caches()
-    info = connector.register_kv_caches(kv, manager_block_size=64, local_block_size=16, tp_rank=1, tp_size=2)
+    info = connector.register_kv_caches(kv, manager_block_size=64, local_block_size=16, tp_rank=1, world_size=2)
     want = []
     for t in kv.values():
         want += [t[0].data_ptr(), t[1].data_ptr()]
     assert info.all_kvcache_ptr_tensor_gpu.tolist() == want
     assert info.kvcache_ptr_tensor_cpu.tolist() == [t.data_ptr() for t in kv.values()]
-    assert info.per_manager_location_spec_shape == (3, 2, 64, 128)
-    assert info.per_manager_location_spec_byte_size == 3 * 2 * 64 * 128 * 2
+    assert info.per_manager_block_shape == (3, 2, 64, 128)
+    assert info.per_manager_block_byte_size == 3 * 2 * 64 * 128 * 2
     assert info.per_token_per_layer_dim_size == 128 and info.local_token_num == 8 * 16
-    assert (info.layer_num, info.tp_rank, info.tp_size, info.dtype) == (3, 1, 2, torch.float16)
+    assert (info.layer_num, info.tp_rank, info.world_size, info.dtype) == (3, 1, 2, torch.float16)
     # V of a layer sits block_num * block_size rows after K: the legacy [2, total, H] view of the same tensor
     assert want[1] - want[0] == 8 * 16 * 128 * 2
 
@@ -154,8 +155,8 @@ def test_register_kv_caches_mla_one_pointer_per_layer():
     kv = {f"l{l}": torch.zeros(32, 128, 576, dtype=torch.uint8) for l in range(4)}
     info = connector.register_kv_caches(kv, manager_block_size=128, local_block_size=128, use_mla=True)
     assert info.all_kvcache_ptr_tensor_gpu.tolist() == [t.data_ptr() for t in kv.values()]
-    assert info.per_manager_location_spec_shape == (4, 1, 128, 576)
-    assert info.per_manager_location_spec_byte_size == 4 * 128 * 576
+    assert info.per_manager_block_shape == (4, 1, 128, 576)
+    assert info.per_manager_block_byte_size == 4 * 128 * 576
     assert info.local_token_num == 32 * 128
 
 
@@ -180,3 +181,137 @@ def test_generate_blocks_idx_bounds_check_runs_on_the_host():
     with pytest.raises(AssertionError):
         connector.generate_blocks_idx([-1], [0, 1, 2, 3], 16, 16, device="cpu")
     assert connector.generate_blocks_idx([], [0], 16, 16, device="cpu").shape == (0, 16)
+
+
+class _FakeCoordinator:
+    """Stands in for TpCoordinatorClient (kv_cache_manager/py_connector/common/tp_coordinator.py): keeps what it is sent."""
+
+    def __init__(self):
+        self.sent = []
+
+    def send(self, data):
+        assert isinstance(data, bytes)
+        self.sent.append(data)
+
+
+class _ExtraConfig:
+    block_per_save_task = 128
+    block_per_load_task = 2
+
+
+def _manager_as_the_connector_builds_it(coordinator):
+    """register_kv_caches' tail, v1_connector.py:416-442: KVCacheInfo and DataTransferManager, all arguments positional."""
+    from tair_kvcache_amd import connector
+    from tair_kvcache_amd.kernel.gather_scatter_helper import CopyBufferAllocator
+    kv = _vllm_caches()
+    ptrs = torch.tensor([t.data_ptr() for t in kv.values()], dtype=torch.int64)
+    all_ptrs = torch.tensor([p for t in kv.values() for p in (t[0].data_ptr(), t[1].data_ptr())], dtype=torch.int64)
+    shape = [3, 2, 16, 128]
+    info = connector.KVCacheInfo(1, 2, kv, ptrs, ptrs, all_ptrs, len(kv), 8 * 16, tuple(shape), 3 * 2 * 16 * 128 * 2, 128,
+                                 torch.device("cpu"), torch.float16)
+    alloc = CopyBufferAllocator(torch.device("cpu"), torch.float16, shape, 4)
+    transfer_client = object()
+    mgr = connector.DataTransferManager(info, 16, alloc, transfer_client, coordinator, _ExtraConfig())
+    return info, mgr
+
+
+def test_kvcache_info_is_the_reference_value_class():
+    # kv_cache_manager/py_connector/common/types.py:9-23: names, order, frozen
+    import dataclasses
+    from tair_kvcache_amd import connector
+    assert [f.name for f in dataclasses.fields(connector.KVCacheInfo)] == [
+        "tp_rank", "world_size", "kvcaches", "kvcache_ptr_tensor_cpu", "kvcache_ptr_tensor_gpu",
+        "all_kvcache_ptr_tensor_gpu", "layer_num", "local_token_num", "per_manager_block_shape",
+        "per_manager_block_byte_size", "per_token_per_layer_dim_size", "device", "dtype"]
+    info, _ = _manager_as_the_connector_builds_it(_FakeCoordinator())
+    with pytest.raises(dataclasses.FrozenInstanceError):
+        info.tp_rank = 0
+
+
+def test_data_transfer_manager_takes_the_reference_constructor_call():
+    # data_transfer.py:47-53 and its call at v1_connector.py:435-442
+    from tair_kvcache_amd import connector
+    params = list(inspect.signature(connector.DataTransferManager.__init__).parameters.values())
+    assert [p.name for p in params[:7]] == ["self", "kvcache_info", "manager_block_size", "copy_buffer_allocator",
+                                            "transfer_client", "coordinator_client", "extra_config"]
+    assert all(p.kind is inspect.Parameter.KEYWORD_ONLY for p in params[7:])
+    coord = _FakeCoordinator()
+    info, mgr = _manager_as_the_connector_builds_it(coord)
+    assert mgr._coordinator_client is coord and isinstance(mgr._extra_config, _ExtraConfig)
+    assert mgr._kvcache_info is info and mgr._manager_block_size == 16
+    assert list(inspect.signature(mgr.create_load_done_callback).parameters) == ["req_id", "tp_rank", "epoch",
+                                                                                 "local_block_ids"]
+    assert list(inspect.signature(mgr.create_save_done_callback).parameters) == ["req_id", "tp_rank", "write_session_id"]
+    mgr.shutdown()
+
+
+def test_load_done_callback_reports_failed_local_blocks_like_start_load_kv():
+    """The loop of start_load_kv (v1_connector.py:448-475) with block_per_load_task = 2 over five blocks: three tasks,
+    the second one fails => the local block ids at positions 2 and 3 are reported (data_transfer.py:172-186)."""
+    import copy
+    import json
+    import math
+    from tair_kvcache_amd import client_types as ct, connector, coordinator_messages as cm
+    coord = _FakeCoordinator()
+    info, mgr = _manager_as_the_connector_builds_it(coord)
+    local_block_ids = [40, 41, 42, 43, 44]
+    block_token_indices = [[b * 16 + i for i in range(16)] for b in local_block_ids]
+    per_task_size = mgr._extra_config.block_per_load_task
+    task_num = math.ceil(len(block_token_indices) / per_task_size)
+    done_callback = mgr.create_load_done_callback("req-7", info.tp_rank, 3, copy.copy(local_block_ids))
+    multi_result = connector.MultiResult(task_num, done_callback)
+    codes = [ct.ClientErrorCode.ER_OK, ct.ClientErrorCode.ER_SDKREAD_ERROR, ct.ClientErrorCode.ER_OK]
+    task_idx = 0
+    for i in range(0, len(block_token_indices), per_task_size):
+        end_idx = min(len(block_token_indices), i + per_task_size)
+        # what load_task submits: the task's code once per block of the task (data_transfer.py:158)
+        assert not coord.sent
+        multi_result.submit_result(task_idx, [codes[task_idx]] * (end_idx - i))
+        task_idx += 1
+    assert len(coord.sent) == 1
+    msg = cm.CoordinateMsgSerializer.loads(coord.sent[0])
+    assert isinstance(msg.content, cm.LoadBlockFinishedEvent)
+    assert (msg.content.request_id, msg.content.tp_rank, msg.content.epoch) == ("req-7", 1, 3)
+    assert msg.content.failed_block_idxs == [42, 43]
+    wire = json.loads(coord.sent[0])
+    assert list(wire) == ["send_time", "content", "create_time"]
+    assert list(wire["content"]) == ["request_id", "tp_rank", "epoch", "failed_block_idxs", "type"]
+    assert wire["content"]["type"] == "LoadBlockFinishedEvent"
+    mgr.shutdown()
+
+
+def test_save_done_callback_reports_one_flag_per_block_like_wait_for_save():
+    """wait_for_save's loop (v1_connector.py:486-519): 300 blocks in tasks of 128 => three tasks; the last one fails."""
+    import json
+    import math
+    from tair_kvcache_amd import client_types as ct, connector, coordinator_messages as cm
+    coord = _FakeCoordinator()
+    info, mgr = _manager_as_the_connector_builds_it(coord)
+    n = 300
+    per_task_size = mgr._extra_config.block_per_save_task
+    task_num = math.ceil(n / per_task_size)
+    multi_result = connector.MultiResult(task_num, mgr.create_save_done_callback("req-9", info.tp_rank, "ws-1"))
+    # tasks finish out of order on the 32-thread pool
+    for task_idx in (2, 0, 1):
+        size = min(n, (task_idx + 1) * per_task_size) - task_idx * per_task_size
+        code = ct.ClientErrorCode.ER_SDKWRITE_ERROR if task_idx == 2 else ct.ClientErrorCode.ER_OK
+        multi_result.submit_result(task_idx, [code] * size)
+    assert len(coord.sent) == 1
+    msg = cm.CoordinateMsgSerializer.loads(coord.sent[0])
+    assert isinstance(msg.content, cm.SendBlockFinishedEvent)
+    assert (msg.content.request_id, msg.content.tp_rank, msg.content.write_session_id) == ("req-9", 1, "ws-1")
+    assert msg.content.is_success_list == [True] * 256 + [False] * 44
+    wire = json.loads(coord.sent[0])
+    assert list(wire["content"]) == ["request_id", "tp_rank", "write_session_id", "is_success_list", "remote_uris", "type"]
+    assert wire["content"]["remote_uris"] == [] and msg.send_time <= msg.create_time + 1.0
+    mgr.shutdown()
+
+
+def test_done_callback_without_a_coordinator_says_so():
+    from tair_kvcache_amd import connector
+    from tair_kvcache_amd.kernel.gather_scatter_helper import CopyBufferAllocator
+    info, _ = _manager_as_the_connector_builds_it(_FakeCoordinator())
+    mgr = connector.DataTransferManager(info, 16, CopyBufferAllocator(torch.device("cpu"), torch.float16, [1], 1), object())
+    with pytest.raises(RuntimeError):
+        mgr.create_save_done_callback("r", 0, "w")([[0]])
+    mgr.shutdown()
