@@ -159,7 +159,8 @@ int32_t kvcm_hip_paged_scatter(const void *const *d_ptr_table, int32_t P, const 
  *    T * row_bytes + trailer_bytes for the packed record;
  *  - trailer: trailer_bytes > 0 appends to every (b, p) tile the bytes
  *    d_trailer_ptr_table[p][d_trailer_idx[b] * trailer_bytes ..] (per-block quantisation scales of an
- *    fp8 cache); on scatter they are written back. No counterpart in the reference, which has only the
+ *    fp8 cache); on scatter they are written back. d_trailer_idx[b] < 0 skips block b's trailers in both directions
+ *    (the staging bytes and the trailer arrays stay as they are). No counterpart in the reference, which has only the
  *    one-pointer-per-layer MLA branch (kv_cache_manager/py_connector/vllm/v1_connector.py:398-403).
  */
 typedef struct kvcm_copy_desc {
@@ -305,6 +306,8 @@ typedef struct kvcm_file_store kvcm_file_store;
  */
 int32_t kvcm_file_store_create(int64_t byte_size_per_block, int64_t bounce_bytes, int32_t sync_on_put,
                                int32_t io_threads, kvcm_file_store **out);
+/* Waits for puts and gets that are still running on other threads to hand back their streams and buffers, then frees
+ * everything. No call may START on a store once its destruction has begun. */
 void kvcm_file_store_destroy(kvcm_file_store *store);
 
 /*

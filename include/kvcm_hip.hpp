@@ -10,8 +10,10 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <condition_variable>
 #include <cstdint>
 #include <cstdlib>
+#include <mutex>
 #include <vector>
 
 #include "kvcm_hip.h"
@@ -113,15 +115,53 @@ inline std::vector<int64_t> ApplyPrefixHash(const std::vector<int64_t> &hash_ids
     return GenKeyVector(hash_ids, 1);
 }
 
-// SdkBufferCheckUtil::GetIovsCrc (kv_cache_manager/client/src/internal/sdk/sdk_buffer_check_util.cu:50-69):
-// cal_byte_size = min(min_cal_byte_size, iovs[0].size / 2); empty result when that is 0 or on error.
-inline std::vector<uint32_t> GetIovsCrc(const std::vector<kvcm_iov_device> &iovs_h, size_t min_cal_byte_size = 4,
-                                        hipStream_t stream = nullptr) {
-    if (iovs_h.empty()) {
+// Number of bytes hashed at each end of an iov: min(min_cal_byte_size, iovs[0].size / 2) -- from the FIRST iov, as
+// kv_cache_manager/client/src/internal/sdk/sdk_buffer_check_util.cu:52 takes it. 0 = nothing to do. Also 0 when any
+// iov has no base address or is shorter than that: the reference would read out of bounds there.
+inline size_t IovCheckBytes(const kvcm_iov_device *iovs_h, size_t n, size_t min_cal_byte_size) {
+    if (n == 0 || !iovs_h) {
+        return 0;
+    }
+    const size_t cal = std::min(min_cal_byte_size, iovs_h[0].size / 2);
+    for (size_t i = 0; i < n && cal > 0; ++i) {
+        if (!iovs_h[i].base || iovs_h[i].size < cal) {
+            return 0;
+        }
+    }
+    return cal;
+}
+
+// SdkBufferCheckUtil::GetIovsCrc on the caller's buffers (sdk_buffer_check_util.cu:50-69, the five-argument form):
+// iovs_d and crcs_d are device arrays with room for iovs_size entries; iovs_h_ptr should be pinned memory (it is
+// read by an asynchronous copy). Allocates nothing on the device. Empty result when there is nothing to hash or on
+// error.
+inline std::vector<uint32_t> GetIovsCrc(const kvcm_iov_device *iovs_h_ptr, size_t iovs_size, kvcm_iov_device *iovs_d,
+                                        uint32_t *crcs_d, hipStream_t stream, size_t min_cal_byte_size = 4) {
+    const size_t cal = IovCheckBytes(iovs_h_ptr, iovs_size, min_cal_byte_size);
+    if (cal == 0 || !iovs_d || !crcs_d || iovs_size > static_cast<size_t>(INT32_MAX)) {
         return {};
     }
-    const size_t cal = std::min(min_cal_byte_size, iovs_h.front().size / 2);
-    if (cal == 0) {
+    if (hipMemcpyAsync(iovs_d, iovs_h_ptr, iovs_size * sizeof(kvcm_iov_device), hipMemcpyHostToDevice, stream) !=
+        hipSuccess) {
+        return {};
+    }
+    if (kvcm_hip_iov_crc32(iovs_d, static_cast<int32_t>(iovs_size), crcs_d, cal, stream) != KVCM_OK) {
+        (void)hipStreamSynchronize(stream);
+        return {};
+    }
+    std::vector<uint32_t> crcs(iovs_size);
+    if (hipMemcpyAsync(crcs.data(), crcs_d, crcs.size() * 4, hipMemcpyDeviceToHost, stream) != hipSuccess ||
+        hipStreamSynchronize(stream) != hipSuccess) {
+        return {};
+    }
+    return crcs;
+}
+
+// The one-argument form (sdk_buffer_check_util.cu:71-87): allocates its device buffers for the call. Call sites that
+// check every transfer take a cell of SdkBufferCheckPool instead.
+inline std::vector<uint32_t> GetIovsCrc(const std::vector<kvcm_iov_device> &iovs_h, size_t min_cal_byte_size = 4,
+                                        hipStream_t stream = nullptr) {
+    if (IovCheckBytes(iovs_h.data(), iovs_h.size(), min_cal_byte_size) == 0) {
         return {};
     }
     detail::DeviceArray<kvcm_iov_device> d_iovs(iovs_h.size());
@@ -129,20 +169,7 @@ inline std::vector<uint32_t> GetIovsCrc(const std::vector<kvcm_iov_device> &iovs
     if (!d_iovs.ptr || !d_crc.ptr) {
         return {};
     }
-    if (hipMemcpyAsync(d_iovs.ptr, iovs_h.data(), iovs_h.size() * sizeof(kvcm_iov_device), hipMemcpyHostToDevice,
-                       stream) != hipSuccess) {
-        return {};
-    }
-    if (kvcm_hip_iov_crc32(d_iovs.ptr, static_cast<int32_t>(iovs_h.size()), d_crc.ptr, cal, stream) != KVCM_OK) {
-        (void)hipStreamSynchronize(stream);
-        return {};
-    }
-    std::vector<uint32_t> crcs(iovs_h.size());
-    if (hipMemcpyAsync(crcs.data(), d_crc.ptr, crcs.size() * 4, hipMemcpyDeviceToHost, stream) != hipSuccess ||
-        hipStreamSynchronize(stream) != hipSuccess) {
-        return {};
-    }
-    return crcs;
+    return GetIovsCrc(iovs_h.data(), iovs_h.size(), d_iovs.ptr, d_crc.ptr, stream, min_cal_byte_size);
 }
 
 // SdkBufferCheckUtil::GetBlocksHash (sdk_buffer_check_util.cc:11-28): one hash per block of iovs_per_block iovs.
@@ -200,6 +227,156 @@ inline int32_t FirstOccurrence(const KeyVector &keys, std::vector<int32_t> *firs
 // owns a kvcm_file_store. One BlockBuffer per block, as kv_cache_manager/client/include/common.h:116-118.
 struct BlockBuffer {
     std::vector<kvcm_iov> iovs;
+};
+using BlockBuffers = std::vector<BlockBuffer>;
+
+// SdkBufferCheckUtil::GetBlocksHash on the caller's buffers (sdk_buffer_check_util.cc:35-61): whole blocks are taken
+// while their iovs fit into max_iov_num (the rest is not checked, :45-47); iovs_h_to_save is host room for
+// max_iov_num entries, pinned in a pool cell. All blocks must hold as many iovs as the first.
+inline std::vector<int64_t> GetBlocksHash(const BlockBuffers &block_buffers, kvcm_iov_device *iovs_d, uint32_t *crcs_d,
+                                          kvcm_iov_device *iovs_h_to_save, size_t max_iov_num, hipStream_t stream,
+                                          size_t min_cal_byte_size = 4) {
+    if (block_buffers.empty() || block_buffers.front().iovs.empty() || !iovs_h_to_save) {
+        return {};
+    }
+    const size_t iov_num = block_buffers.front().iovs.size();
+    size_t n = 0;
+    for (const BlockBuffer &b : block_buffers) {
+        if (b.iovs.size() != iov_num) {
+            return {};
+        }
+        if (n + iov_num > max_iov_num) {
+            break;
+        }
+        for (const kvcm_iov &iov : b.iovs) {
+            iovs_h_to_save[n++] = kvcm_iov_device{iov.base, iov.size};
+        }
+    }
+    const std::vector<uint32_t> crcs = GetIovsCrc(iovs_h_to_save, n, iovs_d, crcs_d, stream, min_cal_byte_size);
+    if (crcs.empty()) {
+        return {};
+    }
+    std::vector<int64_t> out(crcs.size() / iov_num);
+    if (kvcm_blocks_hash_from_crcs(crcs.data(), static_cast<int64_t>(crcs.size()), static_cast<int32_t>(iov_num),
+                                   out.data()) != KVCM_OK) {
+        return {};
+    }
+    return out;
+}
+
+// Reusable buffers for the buffer check, so that checking a transfer allocates nothing:
+// SdkBufferCheckPool (kv_cache_manager/client/src/internal/sdk/sdk_buffer_check_util.h:43-93, .cc:65-132; used at
+// kv_cache_manager/client/src/transfer_client_impl.cc:85-88,129-131,146-148). cell_num cells, each with a pinned host
+// table, a device table, a device CRC array (room for max_check_iov_num iovs) and a non-blocking stream of its own at
+// the default priority. GetCell() blocks until a cell is free; the handle gives the cell back when it goes out of
+// scope.
+class SdkBufferCheckPool {
+public:
+    struct Cell {
+        kvcm_iov_device *h_iovs = nullptr;
+        kvcm_iov_device *d_iovs = nullptr;
+        uint32_t *d_crcs = nullptr;
+        hipStream_t stream = nullptr;
+    };
+
+    class CellHandle {
+    public:
+        CellHandle(SdkBufferCheckPool *pool, Cell *cell) : pool_(pool), cell_(cell) {}
+        CellHandle(CellHandle &&o) noexcept : pool_(o.pool_), cell_(o.cell_) { o.pool_ = nullptr, o.cell_ = nullptr; }
+        CellHandle(const CellHandle &) = delete;
+        CellHandle &operator=(const CellHandle &) = delete;
+        ~CellHandle() {
+            if (pool_ && cell_) {
+                pool_->PutCell(cell_);
+            }
+        }
+        Cell *operator->() { return cell_; }
+        Cell &operator*() { return *cell_; }
+        explicit operator bool() const { return cell_ != nullptr; }
+
+    private:
+        SdkBufferCheckPool *pool_;
+        Cell *cell_;
+    };
+
+    explicit SdkBufferCheckPool(size_t cell_num = 4) : cells_(cell_num) {}
+    SdkBufferCheckPool(const SdkBufferCheckPool &) = delete;
+    SdkBufferCheckPool &operator=(const SdkBufferCheckPool &) = delete;
+    ~SdkBufferCheckPool() {
+        for (Cell &c : cells_) {
+            if (c.stream) {
+                (void)hipStreamSynchronize(c.stream);
+                (void)hipStreamDestroy(c.stream);
+            }
+            if (c.h_iovs) {
+                (void)hipHostFree(c.h_iovs);
+            }
+            if (c.d_iovs) {
+                (void)hipFree(c.d_iovs);
+            }
+            if (c.d_crcs) {
+                (void)hipFree(c.d_crcs);
+            }
+        }
+    }
+
+    // Allocates every cell on the current device. false = some allocation failed (what exists is freed by the
+    // destructor); the pool then hands out no cells it could not fill.
+    bool Init(size_t max_check_iov_num) {
+        if (max_check_iov_num == 0 || !free_.empty()) {
+            return false;
+        }
+        max_iov_num_ = max_check_iov_num;
+        const size_t iov_bytes = max_check_iov_num * sizeof(kvcm_iov_device), crc_bytes = max_check_iov_num * 4;
+        for (Cell &c : cells_) {
+            if (hipHostMalloc(reinterpret_cast<void **>(&c.h_iovs), iov_bytes, hipHostMallocDefault) != hipSuccess ||
+                hipMalloc(reinterpret_cast<void **>(&c.d_iovs), iov_bytes) != hipSuccess ||
+                hipMalloc(reinterpret_cast<void **>(&c.d_crcs), crc_bytes) != hipSuccess ||
+                hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking) != hipSuccess) {
+                free_.clear();
+                return false;
+            }
+            free_.push_back(&c);
+        }
+        return true;
+    }
+
+    CellHandle GetCell() {
+        std::unique_lock<std::mutex> lock(mutex_);
+        cv_.wait(lock, [this] { return !free_.empty(); });
+        Cell *c = free_.back();
+        free_.pop_back();
+        return CellHandle(this, c);
+    }
+
+    // GetBlocksHash of `block_buffers` on a cell of this pool: what the transfer client does around every transfer
+    // when KVCM_SDK_CHECK is set (transfer_client_impl.cc:127-133).
+    std::vector<int64_t> GetBlocksHash(const BlockBuffers &block_buffers, size_t min_cal_byte_size = 4) {
+        CellHandle cell = GetCell();
+        return kvcm::GetBlocksHash(block_buffers, cell->d_iovs, cell->d_crcs, cell->h_iovs, max_iov_num_, cell->stream,
+                                   min_cal_byte_size);
+    }
+
+    size_t FreeCells() {
+        std::lock_guard<std::mutex> lock(mutex_);
+        return free_.size();
+    }
+    size_t MaxCheckIovNum() const { return max_iov_num_; }
+
+private:
+    void PutCell(Cell *c) {
+        {
+            std::lock_guard<std::mutex> lock(mutex_);
+            free_.push_back(c);
+        }
+        cv_.notify_one();
+    }
+
+    std::mutex mutex_;
+    std::condition_variable cv_;
+    std::vector<Cell> cells_;
+    std::vector<Cell *> free_;
+    size_t max_iov_num_ = 0;
 };
 
 class LocalFileStore {

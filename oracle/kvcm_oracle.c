@@ -343,7 +343,7 @@ static void copy_one_block(const kvcm_ref_copy_desc *d, int32_t b, int scatter) 
                 memcpy(st, row, (size_t)run_bytes);
             }
         }
-        if (d->trailer_bytes > 0) {
+        if (d->trailer_bytes > 0 && d->trailer_idx[b] >= 0) { /* a negative trailer index skips the trailer */
             uint8_t *tr = (uint8_t *)d->trailer_ptr_table[p] + (int64_t)d->trailer_idx[b] * d->trailer_bytes;
             uint8_t *st = tile + (int64_t)d->T * d->row_bytes;
             if (scatter) {

@@ -32,6 +32,10 @@ def get_iovs_crc(iovs: Sequence[IovLike], device="cuda", cal_byte_size: Optional
     if cal == 0:
         return []
     n = len(iovs)
+    for i, (base, size) in enumerate(iovs):
+        # the count of bytes comes from the first iov only; the reference would read past a shorter iov's end
+        if int(base) == 0 or int(size) < cal:
+            raise ValueError(f"iov {i} (base {int(base):#x}, size {int(size)}) cannot supply {cal} bytes per end")
     table = (_lib.IovDevice * n)(*[_lib.IovDevice(int(b), int(s)) for b, s in iovs])
     raw = torch.frombuffer(bytearray(bytes(table)), dtype=torch.uint8)
     d_iovs = raw.to(device)

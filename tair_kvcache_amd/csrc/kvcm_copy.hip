@@ -247,8 +247,9 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
                     pp[u] = pool + slot * a.row_bytes + static_cast<int64_t>(off) * CS;
                     sp[u] = tile + static_cast<int64_t>(cc) * CS;
                 }
-                if (a.trailer_bytes > 0 && cc == 0) {
-                    // the thread that owns a tile's first chunk also moves the tile's trailer
+                if (a.trailer_bytes > 0 && cc == 0 && trailer_idx[b] >= 0) {
+                    // the thread that owns a tile's first chunk also moves the tile's trailer (a negative trailer
+                    // index means "no trailer for this block": nothing is read or written)
                     unsigned char *tr = static_cast<unsigned char *>(const_cast<void *>(trailer_table[p])) +
                                         static_cast<int64_t>(trailer_idx[b]) * a.trailer_bytes;
                     unsigned char *st = tile + a.tile_payload;
@@ -421,7 +422,8 @@ int32_t launch_copy(const kvcm_copy_desc *d, bool scatter, hipStream_t stream) {
     a.div_run = make_fastdiv(a.chunks_per_run);
     a.div_entry = make_fastdiv(a.ptrs_per_entry);
     a.div_units = make_fastdiv(a.units_per_block);
-    a.xcd_remap = env_int("KVCM_COPY_XCD_REMAP", 1);
+    static const int xcd_remap = env_int("KVCM_COPY_XCD_REMAP", 1);  // tuning knob, read once per process
+    a.xcd_remap = xcd_remap;
 
     int64_t grid = units;
     if (d->max_workgroups > 0) {

@@ -202,7 +202,7 @@ struct kvcm_file_store {
             destroy(lane);
             lock.lock();
             lanes_alive--;
-            lane_freed.notify_one();
+            lane_freed.notify_all();
             return kvcm::hip_code(e);
         }
         *out = lane;
@@ -212,7 +212,7 @@ struct kvcm_file_store {
     void release(kvcm::Lane *lane) {
         std::lock_guard<std::mutex> lock(mu);
         idle.push_back(lane);
-        lane_freed.notify_one();
+        lane_freed.notify_all();  // a caller waiting for a lane, and the destroyer waiting for all of them
     }
 
     static void destroy(kvcm::Lane *lane) {
@@ -442,8 +442,15 @@ void kvcm_file_store_destroy(kvcm_file_store *store) {
         return;
     }
     store->stop_pool();
-    for (kvcm::Lane *lane : store->idle) {
-        kvcm_file_store::destroy(lane);
+    {
+        // a put or get that is still running holds its lane: wait until every lane is back before freeing them
+        std::unique_lock<std::mutex> lock(store->mu);
+        store->lane_freed.wait(lock, [store] { return static_cast<int>(store->idle.size()) == store->lanes_alive; });
+        for (kvcm::Lane *lane : store->idle) {
+            kvcm_file_store::destroy(lane);
+        }
+        store->idle.clear();
+        store->lanes_alive = 0;
     }
     delete store;
 }

@@ -19,6 +19,7 @@
 // dependent-instruction latency of the chain wave, which no amount of bandwidth removes.
 #include "kvcm_internal.h"
 
+#include <atomic>
 #include <cstdlib>
 
 namespace kvcm {
@@ -527,6 +528,12 @@ __global__ __launch_bounds__(256) void iov_crc32_kernel(const kvcm_iov_device *_
     }
     const uint8_t *p = static_cast<const uint8_t *>(iovs[i].base);
     const size_t size = iovs[i].size;
+    if (!p || size < cal_bytes) {
+        // cal_bytes comes from the first iov only: an iov without an address, or shorter than that, is not read at
+        // all and gets the value 0 (the reference reads out of bounds here)
+        out[i] = 0;
+        return;
+    }
     uint32_t crc = 0xFFFFFFFFu;
     for (size_t k = 0; k < cal_bytes; ++k) {
         crc = crc32_byte(crc, p[k]);
@@ -536,6 +543,14 @@ __global__ __launch_bounds__(256) void iov_crc32_kernel(const kvcm_iov_device *_
     }
     out[i] = ~crc;
 }
+
+// Test hook: non-zero makes every launch take the loader path that a workgroup spanning >= 4 GiB of tokens would take.
+// Starts from the environment variable KVCM_HASH_FORCE_GLOBAL_LOADS (read once, when the library is loaded) and is
+// switched by kvcm_test_hook_hash_force_global_loads, which no header declares.
+std::atomic<int32_t> g_force_global_loads{[] {
+    const char *fg = std::getenv("KVCM_HASH_FORCE_GLOBAL_LOADS");
+    return (fg && fg[0] == '1') ? 1 : 0;
+}()};
 
 template <typename TokT>
 int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_t R, int32_t block_size, int64_t seed,
@@ -550,9 +565,7 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
         return KVCM_ERR_INVALID_ARG;
     }
     const dim3 grid(static_cast<uint32_t>((static_cast<int64_t>(R) + kReqs - 1) / kReqs));
-    // test hook: take the loader path that a workgroup spanning >= 4 GiB of tokens would take
-    const char *fg = std::getenv("KVCM_HASH_FORCE_GLOBAL_LOADS");
-    const int32_t force_global = (fg && fg[0] == '1') ? 1 : 0;
+    const int32_t force_global = g_force_global_loads.load(std::memory_order_relaxed);
 #define KVCM_LAUNCH_HASH(CHUNK, BS)                                                                                  \
     hipLaunchKernelGGL((hash_tokens_kernel<TokT, CHUNK, BS>), grid, dim3(kThreads), 0, stream, d_tokens,            \
                        d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
@@ -583,6 +596,11 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
 extern "C" {
 
 int32_t kvcm_hip_version(void) { return 100; }
+
+// For the parity tests only (not part of the C-ABI): returns the previous setting.
+int32_t kvcm_test_hook_hash_force_global_loads(int32_t on) {
+    return kvcm::g_force_global_loads.exchange(on ? 1 : 0, std::memory_order_relaxed);
+}
 
 const char *kvcm_hip_error_string(int32_t code) {
     switch (code) {

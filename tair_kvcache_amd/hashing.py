@@ -24,10 +24,19 @@ def _offsets_for(tokens, token_offsets):
         R, L = tokens.shape
         off = torch.arange(R + 1, dtype=torch.int64, device=tokens.device) * L
         return off, R
-    require_cuda(token_offsets, "token_offsets")
-    if token_offsets.dtype != torch.int64 or token_offsets.dim() != 1 or token_offsets.numel() < 1:
-        raise ValueError("token_offsets must be a 1-D int64 tensor of R+1 entries")
+    _require_offsets(token_offsets, "token_offsets", tokens.device)
     return token_offsets.contiguous(), token_offsets.numel() - 1
+
+
+def _require_offsets(t, name, device, entries=None):
+    """Offsets are read by the kernel as they are: int64, 1-D, on the tokens' device, R+1 entries."""
+    require_cuda(t, name)
+    if t.dtype != torch.int64 or t.dim() != 1 or t.numel() < 1:
+        raise ValueError(f"{name} must be a 1-D int64 tensor of R+1 entries")
+    if t.device != device:
+        raise ValueError(f"{name} is on {t.device}, the tokens on {device}")
+    if entries is not None and t.numel() != entries:
+        raise ValueError(f"{name} has {t.numel()} entries, expected {entries}")
 
 
 def hash_tokens(tokens: torch.Tensor, block_size: int, token_offsets: Optional[torch.Tensor] = None,
@@ -48,6 +57,16 @@ def hash_tokens(tokens: torch.Tensor, block_size: int, token_offsets: Optional[t
         raise ValueError("block_size must be positive")
     tokens = tokens.contiguous()
     off, R = _offsets_for(tokens, token_offsets)
+    if key_offsets is not None:
+        _require_offsets(key_offsets, "key_offsets", tokens.device, R + 1)
+        key_offsets = key_offsets.contiguous()
+    if keys is not None:
+        require_cuda(keys, "keys")
+        if keys.dtype != torch.int64 or keys.device != tokens.device or not keys.is_contiguous():
+            raise ValueError("keys must be a contiguous int64 tensor on the tokens' device")
+        if token_offsets is None and keys.numel() < R * (tokens.shape[1] // int(block_size)):
+            raise ValueError(f"keys holds {keys.numel()} entries, the batch yields "
+                             f"{R * (tokens.shape[1] // int(block_size))}")
     if key_offsets is None:
         counts = (off[1:] - off[:-1]) // int(block_size)
         key_offsets = torch.zeros(R + 1, dtype=torch.int64, device=tokens.device)
@@ -89,6 +108,9 @@ def apply_prefix_hash(hash_ids: torch.Tensor, offsets: Optional[torch.Tensor] = 
     ids = hash_ids.contiguous().reshape(-1)
     if offsets is None:
         offsets = torch.tensor([0, ids.numel()], dtype=torch.int64, device=ids.device)
+    else:
+        _require_offsets(offsets, "offsets", ids.device)
+        offsets = offsets.contiguous()
     keys = torch.empty_like(ids)
     rc = lib().kvcm_hip_prefix_chain(ptr(ids), ptr(offsets), offsets.numel() - 1, ptr(keys),
                                      stream_handle(ids.device))

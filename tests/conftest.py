@@ -39,3 +39,23 @@ def golden():
     import json
     with open(os.path.join(ROOT, "tests", "golden", "hash_golden.json")) as f:
         return json.load(f)
+
+
+@pytest.fixture
+def force_general_hash_loader():
+    """Switches the block-key kernel to the loader form it uses when a workgroup's requests span 4 GiB or more, through
+    the library's test hook (an exported symbol that no header declares); restores the previous setting afterwards."""
+    import ctypes
+    from tair_kvcache_amd import _lib
+    hook = _lib.lib().kvcm_test_hook_hash_force_global_loads
+    hook.restype, hook.argtypes = ctypes.c_int32, [ctypes.c_int32]
+    state = {"previous": None}
+
+    def switch(on):
+        previous = hook(1 if on else 0)
+        if state["previous"] is None:
+            state["previous"] = previous
+
+    yield switch
+    if state["previous"] is not None:
+        hook(state["previous"])

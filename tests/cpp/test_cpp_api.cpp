@@ -7,7 +7,9 @@
 #include <cstdlib>
 #include <cstring>
 #include <random>
+#include <atomic>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "kvcm_hip.hpp"
@@ -255,6 +257,88 @@ static void test_first_occurrence() {
     EXPECT(kvcm::FirstOccurrence({}, &none) == KVCM_OK && none.empty());
 }
 
+// SdkBufferCheckPool as the reference's tests use it
+// (kv_cache_manager/client/src/internal/sdk/test/sdk_buffer_check_util_test.cc:283-382): equal buffers give equal
+// block hashes through a cell, cells are handed out and taken back, eight threads share four cells.
+static kvcm::BlockBuffer four_iov_block(char fill, size_t byte_size = 4 * 1024) {
+    char *buffer = nullptr;
+    EXPECT(hipMalloc(reinterpret_cast<void **>(&buffer), byte_size) == hipSuccess);
+    std::string init(byte_size, fill);
+    (void)hipMemcpy(buffer, init.data(), byte_size, hipMemcpyHostToDevice);
+    kvcm::BlockBuffer b;
+    for (int i = 0; i < 4; ++i) {
+        b.iovs.push_back(kvcm_iov{KVCM_MEMORY_GPU, 0, buffer + 1024 * i, 1024});
+    }
+    return b;
+}
+
+static void test_buffer_check_pool() {
+    const size_t max_check_iov_num = 10;
+    {
+        kvcm::SdkBufferCheckPool pool;
+        EXPECT(pool.Init(max_check_iov_num));
+        kvcm::BlockBuffers blocks{four_iov_block('a'), four_iov_block('a'), four_iov_block('a')};
+        auto handle = pool.GetCell();
+        auto hashes = kvcm::GetBlocksHash(blocks, handle->d_iovs, handle->d_crcs, handle->h_iovs, max_check_iov_num,
+                                          handle->stream);
+        EXPECT(hashes.size() == 2);  // the third block's iovs would exceed max_check_iov_num: not checked
+        EXPECT(hashes.size() == 2 && hashes[0] == hashes[1]);
+        // the value: CRC of "aaaa" + "aaaa" per iov, chained over four iovs, from the oracle
+        std::string a(1024, 'a');
+        kvcm_ref_iov ref[4] = {{a.data(), 1024}, {a.data(), 1024}, {a.data(), 1024}, {a.data(), 1024}};
+        uint32_t crcs[4];
+        int64_t want[1];
+        kvcm_ref_iov_crc32(ref, 4, crcs, 4);
+        kvcm_ref_blocks_hash_from_crcs(crcs, 4, 4, want);
+        EXPECT(!hashes.empty() && hashes[0] == want[0]);
+        // an iov shorter than the bytes taken per end, or without an address: nothing is launched
+        kvcm::BlockBuffers bad{four_iov_block('a')};
+        bad[0].iovs[2].size = 3;
+        EXPECT(kvcm::GetBlocksHash(bad, handle->d_iovs, handle->d_crcs, handle->h_iovs, max_check_iov_num,
+                                   handle->stream).empty());
+        bad[0].iovs[2].size = 1024;
+        bad[0].iovs[1].base = nullptr;
+        EXPECT(kvcm::GetBlocksHash(bad, handle->d_iovs, handle->d_crcs, handle->h_iovs, max_check_iov_num,
+                                   handle->stream).empty());
+    }
+    {
+        kvcm::SdkBufferCheckPool pool(2);
+        EXPECT(pool.Init(max_check_iov_num));
+        EXPECT(pool.FreeCells() == 2);
+        {
+            auto h1 = pool.GetCell();
+            EXPECT(pool.FreeCells() == 1);
+            auto h2 = pool.GetCell();
+            EXPECT(pool.FreeCells() == 0);
+            EXPECT(h1->d_iovs != h2->d_iovs && h1->stream != h2->stream);
+        }
+        EXPECT(pool.FreeCells() == 2);
+    }
+    {
+        kvcm::SdkBufferCheckPool pool;
+        EXPECT(pool.Init(max_check_iov_num));
+        std::vector<kvcm::BlockBuffers> sets{{four_iov_block('a')}, {four_iov_block('a')}};
+        const auto expect = pool.GetBlocksHash(sets[0]);
+        EXPECT(expect.size() == 1);
+        std::atomic<int> wrong{0};
+        for (int round = 0; round < 20; ++round) {
+            std::vector<std::thread> threads;
+            for (int j = 0; j < 8; ++j) {
+                threads.emplace_back([&, round] {
+                    if (pool.GetBlocksHash(sets[round % 2]) != expect) {
+                        wrong.fetch_add(1);
+                    }
+                });
+            }
+            for (auto &t : threads) {
+                t.join();
+            }
+        }
+        EXPECT(wrong.load() == 0);
+        EXPECT(pool.FreeCells() == 4);
+    }
+}
+
 int main() {
     int n = 0;
     if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
@@ -267,6 +351,7 @@ int main() {
     test_gather_scatter_c_abi();
     test_local_file_put_get_with_gpu();
     test_first_occurrence();
+    test_buffer_check_pool();
     std::printf("%d checks, %d failed\n", g_run, g_failed);
     return g_failed == 0 ? 0 : 1;
 }

@@ -232,6 +232,32 @@ def test_mla_fp8_with_interleaved_scales(oracle):
         assert not g[rest].any()
         gs = host(scales2[l], np.float32)
         assert (gs[blocks] == scales[l][blocks]).all() and not gs[rest].any()
+    # a negative trailer index skips a block's trailers, a negative run start its rows: against the oracle, both ways
+    tr_np = blocks.astype(np.int32).copy()
+    tr_np[[0, 3]] = -1
+    runs_np = (blocks * T).astype(np.int32)
+    runs_np[[3, 5]] = -1
+    want2 = np.full((B, L * rec), 0xEE, dtype=np.uint8)
+    d, keep = oracle.make_desc(pools, want2, runs_np, None, B, T, row, run_tokens=T, trailers=scales, trailer_idx=tr_np,
+                               trailer_bytes=4)
+    oracle.gather_ex(d)
+    st.fill_(0xEE)
+    run_start, tr_idx = dev(runs_np), dev(tr_np)
+    assert _lib.lib().kvcm_hip_gather_ex(desc(table, ttable), torch.cuda.current_stream().cuda_stream) == 0
+    sync()
+    assert (host(st, np.uint8) == want2).all()
+    w_pools, w_scales = [np.zeros_like(p) for p in pools], [np.zeros_like(x) for x in scales]
+    d, keep = oracle.make_desc(w_pools, want2, runs_np, None, B, T, row, run_tokens=T, trailers=w_scales,
+                               trailer_idx=tr_np, trailer_bytes=4)
+    oracle.scatter_ex(d)
+    pools3 = [torch.zeros_like(t) for t in d_pools]
+    scales3 = [torch.zeros_like(t) for t in d_scales]
+    assert _lib.lib().kvcm_hip_scatter_ex(desc(ptr_table(pools3), ptr_table(scales3)),
+                                          torch.cuda.current_stream().cuda_stream) == 0
+    sync()
+    for l in range(L):
+        assert (host(pools3[l], np.uint8) == w_pools[l]).all()
+        assert host(scales3[l], np.float32).tobytes() == w_scales[l].tobytes()
 
 
 def test_legacy_single_block_operators(oracle):

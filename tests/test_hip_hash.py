@@ -79,10 +79,10 @@ def test_ragged_batch_and_seed(oracle):
 
 
 @pytest.mark.parametrize("dtype", [np.int64, np.int32])
-def test_general_loader_path(oracle, monkeypatch, dtype):
+def test_general_loader_path(oracle, force_general_hash_loader, dtype):
     """The loader form used when a workgroup's requests span 4 GiB or more (32-bit buffer offsets cannot reach),
     forced here through its test hook, on a ragged batch whose last request ends exactly at the end of the buffer."""
-    monkeypatch.setenv("KVCM_HASH_FORCE_GLOBAL_LOADS", "1")
+    force_general_hash_loader(True)
     rng = np.random.default_rng(17)
     lens = [int(x) for x in rng.integers(0, 900, size=150)] + [64]
     flat = rng.integers(-2**31, 2**31 - 1, size=sum(lens), dtype=np.int64).astype(dtype)
@@ -134,3 +134,28 @@ def test_sha256_keys(oracle):
     keys, n_prefix, n_new = _h().prepare_block_keys(strs[10:20], prefix_keys=strs[:3])
     assert (n_prefix, n_new) == (3, 10) and keys == want[:3] + want[10:20]
     assert _h().prepare_block_keys([], None) == ([], 0, 0)
+
+
+def test_bad_buffers_are_refused_on_the_host():
+    """Short key buffers, offsets of the wrong type, length or device would be out-of-bounds device accesses: ValueError."""
+    h = _h()
+    tok = torch.zeros(4, 64, dtype=torch.int64, device="cuda")
+    with pytest.raises(ValueError):
+        h.hash_tokens(tok, 16, keys=torch.empty(15, dtype=torch.int64, device="cuda"))       # 16 keys needed
+    with pytest.raises(ValueError):
+        h.hash_tokens(tok, 16, keys=torch.empty(16, dtype=torch.int32, device="cuda"))
+    with pytest.raises(ValueError):
+        h.hash_tokens(tok, 16, keys=torch.empty(16, dtype=torch.int64))                      # keys on the host
+    flat = tok.reshape(-1)
+    off = torch.arange(5, dtype=torch.int64, device="cuda") * 64
+    with pytest.raises(ValueError):
+        h.hash_tokens(flat, 16, token_offsets=off.cpu())
+    with pytest.raises(ValueError):
+        h.hash_tokens(flat, 16, token_offsets=off.to(torch.int32))
+    with pytest.raises(ValueError):
+        h.hash_tokens(flat, 16, token_offsets=off, key_offsets=torch.zeros(4, dtype=torch.int64, device="cuda"))
+    with pytest.raises(ValueError):
+        h.apply_prefix_hash(flat, offsets=torch.tensor([0, 256], dtype=torch.int64))         # offsets on the host
+    keys, _ = h.hash_tokens(flat, 16, token_offsets=off)                                     # and the good call works
+    sync()
+    assert keys.numel() == 16

@@ -27,9 +27,9 @@ def _case(rng):
 
 
 @pytest.mark.parametrize("force_global", ["0", "1"])
-def test_random_batches(oracle, monkeypatch, force_global):
+def test_random_batches(oracle, force_general_hash_loader, force_global):
     from tair_kvcache_amd import hashing
-    monkeypatch.setenv("KVCM_HASH_FORCE_GLOBAL_LOADS", force_global)
+    force_general_hash_loader(force_global == "1")
     rng = np.random.default_rng(77 + int(force_global))
     for i in range(70 if force_global == "0" else 30):
         R, lens, bs, seed, dtype = _case(rng)

@@ -315,3 +315,16 @@ def test_done_callback_without_a_coordinator_says_so():
     with pytest.raises(RuntimeError):
         mgr.create_save_done_callback("r", 0, "w")([[0]])
     mgr.shutdown()
+
+
+def test_hashing_and_buffer_check_reject_bad_arguments_before_any_launch():
+    from tair_kvcache_amd import buffer_check, hashing
+    with pytest.raises(ValueError):
+        hashing.hash_tokens(torch.zeros(2, 32, dtype=torch.int64), 16)             # tokens not on the GPU
+    with pytest.raises(ValueError):
+        hashing.apply_prefix_hash(torch.zeros(8, dtype=torch.int64))
+    with pytest.raises(ValueError):   # an iov shorter than the bytes taken from the first iov's size
+        buffer_check.get_iovs_crc([(0x1000, 64), (0x2000, 3)], device="cpu")
+    with pytest.raises(ValueError):   # an iov without an address
+        buffer_check.get_iovs_crc([(0x1000, 64), (0, 64)], device="cpu")
+    assert buffer_check.get_iovs_crc([(0x1000, 1)], device="cpu") == []            # size 1 -> nothing to hash

@@ -210,3 +210,37 @@ def test_threaded_copy_equals_serial(oracle):
     d2, keep2 = oracle.make_desc(pools, b, tidx, None, 40, T, D * 2)
     oracle.gather_ex(d2, threads=4)
     assert (a == b).all()
+
+
+def test_trailer_is_skipped_for_negative_trailer_index_bruteforce(oracle):
+    """trailer_idx[b] < 0 = no trailer for block b: on gather its staging trailer bytes keep their fill, on scatter no
+    scale is written; a block whose rows are skipped (run start < 0) still moves its trailer when the index is valid."""
+    L, T, row, nblocks = 3, 4, 16, 8
+    rng = np.random.default_rng(8)
+    pools = [rng.integers(0, 254, size=(nblocks * T, row), dtype=np.uint8) for _ in range(L)]
+    scales = [rng.standard_normal(nblocks).astype(np.float32) for _ in range(L)]
+    runs = np.array([5 * T, -1, 2 * T], dtype=np.int32)      # block 1: rows skipped
+    tr_idx = np.array([-1, 6, 2], dtype=np.int32)              # block 0: trailer skipped
+    rec = T * row + 4
+    st = np.full((3, L * rec), 0xEE, dtype=np.uint8)
+    d, keep = oracle.make_desc(pools, st, runs, None, 3, T, row, run_tokens=T, trailers=scales, trailer_idx=tr_idx,
+                               trailer_bytes=4)
+    oracle.gather_ex(d)
+    for l in range(L):
+        base = l * rec
+        assert (st[0, base:base + T * row] == pools[l][5 * T:6 * T].reshape(-1)).all()
+        assert (st[0, base + T * row:base + rec] == 0xEE).all()                              # no trailer moved
+        assert (st[1, base:base + T * row] == 0xEE).all()                                    # rows skipped
+        assert st[1, base + T * row:base + rec].tobytes() == scales[l][6:7].tobytes()        # trailer still moved
+        assert st[2, base + T * row:base + rec].tobytes() == scales[l][2:3].tobytes()
+    pools2 = [np.zeros_like(p) for p in pools]
+    scales2 = [np.zeros_like(s) for s in scales]
+    d, keep = oracle.make_desc(pools2, st, runs, None, 3, T, row, run_tokens=T, trailers=scales2, trailer_idx=tr_idx,
+                               trailer_bytes=4)
+    oracle.scatter_ex(d)
+    for l in range(L):
+        assert scales2[l][6] == scales[l][6] and scales2[l][2] == scales[l][2]
+        assert not np.delete(scales2[l], [6, 2]).any()
+        for blk in (5, 2):
+            assert (pools2[l][blk * T:(blk + 1) * T] == pools[l][blk * T:(blk + 1) * T]).all()
+        assert not np.delete(pools2[l].reshape(nblocks, -1), [5, 2], axis=0).any()
