@@ -9,11 +9,17 @@ One "step" = one pass of the hot path over one batch of synthetic input, inputs 
 `value` = algorithmic bytes of one step / wall time of one step, in GB/s (1e9). Per-kernel durations come from
 events recorded on the launch stream inside the timed region.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--pool-blocks N] [--no-cpu-baseline]
+After the timed steps the same process measures, outside `value`: the block-key kernel at other chain counts, the
+reference-signature call (Python-list indices, one transfer task of 128 blocks, index upload inside the timed
+region), the kernel on one contiguous buffer (the chip's own read+write ceiling), the other four benchmark
+configurations at their full sizes (key `configs`), and the CPU path on this host's cores (key `cpu_baseline`).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--pool-blocks N] [--no-cpu-baseline] [--no-configs]
 
 Prints ONE JSON line. Runs on one GPU only.
 """
 import argparse
+import hashlib
 import json
 import os
 import sys
@@ -25,17 +31,54 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
-# HBM bytes per launch of the two copy kernels at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# scaled by a plain 8 GiB copy in the same run (profiles/copy_span_llama3_8b_hbm_traffic.md). Counters cannot be read
-# from inside this process, so the figures are carried here and reported only for the workload they were taken on.
-MEASURED_TRAFFIC = {"unique_blocks": 12416, "gather": 52077746636, "scatter": 52079466648,
-                    "hash_saturated": int((512.6 + 38.4) * 2**20)}
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain 8 GiB copy in the same run
+# (profiles/copy_span_llama3_8b_hbm_traffic.md, profiles/hash_tokens_16384_chains_hbm_traffic.md). Counters cannot be
+# read from inside this process, so the figures are carried here together with the digest of the kernel sources they
+# were measured on: a run whose sources differ reports traffic null and says why.
+KERNEL_SOURCES = ("tair_kvcache_amd/csrc/kvcm_copy.hip", "tair_kvcache_amd/csrc/kvcm_hash.hip",
+                  "tair_kvcache_amd/csrc/kvcm_internal.h")
+MEASURED_TRAFFIC = {"sources_sha256": "unset", "unique_blocks": 12416, "gather": 52077746636,
+                    "scatter": 52079466648, "hash_saturated": int((512.6 + 40.1) * 2**20)}
 
 # Llama-3-8B KV layout: the configuration the headline metric is quoted on
 LAYERS, KV_HEADS, HEAD_DIM, ITEMSIZE = 32, 8, 128, 2
 T = 16
 REQUESTS, TOKENS_PER_REQ, VOCAB = 64, 4096, 128256
 SHARED_REQS, SHARED_TOKENS = 32, 2048
+TASK_BLOCKS = 128  # block_per_save_task / block_per_load_task of the reference connector (vllm/config.py:23-24)
+
+# Dependent VALU instructions of one wave issue 3.65 ns apart on this chip (measured) and one step of the recurrence
+# is three of them deep, so one request of n tokens cannot be hashed in less than n x 10.95 ns.
+HASH_STEP_FLOOR_NS = 10.95
+
+
+def kernel_sources_digest():
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def zipf_prefix_tokens(np, requests=1024, length=1024, vocab=152064, block=16, templates=16, s=1.2, seed=0):
+    """Token IDs of the page-size-1 configuration: every request starts with a prefix of one of `templates` shared
+    sequences and goes on with tokens of its own. The template is drawn Zipf(s) over the template ranks and the prefix
+    length Zipf(s) over 4, 8, 12, ... blocks (capped at the request), so a few prefixes are shared by many requests
+    and most shared prefixes are short. Returns (tokens int64 [requests, length], template id, prefix length)."""
+    rng = np.random.default_rng(seed)
+    tok = rng.integers(0, vocab, size=(requests, length), dtype=np.int64)
+    shared = rng.integers(0, vocab, size=(templates, length), dtype=np.int64)
+    ranks = np.arange(1, templates + 1, dtype=np.float64)
+    p_template = ranks ** -s / np.sum(ranks ** -s)
+    which = rng.choice(templates, size=requests, p=p_template)
+    max_units = length // (4 * block)
+    units = np.arange(1, max_units + 1, dtype=np.float64)
+    p_len = units ** -s / np.sum(units ** -s)
+    plen = rng.choice(max_units, size=requests, p=p_len) + 1
+    plen = plen * 4 * block
+    for r in range(requests):
+        tok[r, :plen[r]] = shared[which[r], :plen[r]]
+    return tok, which, plen
 
 
 def build_inputs(torch, np, pool_blocks, device):
@@ -67,7 +110,170 @@ def build_inputs(torch, np, pool_blocks, device):
                 save_blocks=save_blocks, load_blocks=load_blocks)
 
 
-def cpu_baseline(np, O, cores):
+def gpu_ms(torch, fn, reps, warm=2):
+    """Average milliseconds of one call of fn, from events on the stream the kernels are launched on."""
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def copy_figures(ms, nbytes):
+    gbps = nbytes / (ms * 1e-3) / 1e9
+    return {"ms": round(ms, 4), "GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4)}
+
+
+def hash_figures(torch, hashing, tokens, block, reps):
+    R, L = tokens.shape
+    toff = torch.arange(R + 1, dtype=torch.int64, device=tokens.device) * L
+    koff = torch.arange(R + 1, dtype=torch.int64, device=tokens.device) * (L // block)
+    keys = torch.empty(R * (L // block), dtype=torch.int64, device=tokens.device)
+    ms = gpu_ms(torch, lambda: hashing.hash_tokens(tokens, block, token_offsets=toff, keys=keys, key_offsets=koff), reps)
+    return keys, {"hash_chains": R, "tokens_per_chain": L, "block_tokens": block, "keys": keys.numel(),
+                  "hash_ms": round(ms, 4), "keys_per_s": round(keys.numel() / (ms * 1e-3)),
+                  "hash_floor_ms": round(L * HASH_STEP_FLOOR_NS * 1e-6, 4)}
+
+
+def other_configs(torch, np, device, reps=5):
+    """BASELINE configurations 1, 3, 4 and 5 at their full sizes, one after the other (memory is released in between):
+    save (gather) and load (scatter) milliseconds, GB/s of read+written bytes and the fraction of the HBM peak, and the
+    block-key kernel at the configuration's own request count. A sample of every result is checked on the device."""
+    from tair_kvcache_amd import _lib, hashing, save_selection
+    from tair_kvcache_amd.kernel import batch_gather_scatter_helper as bgs
+    out = {}
+
+    def release():
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+
+    def tokens_uniform(R, L, vocab, seed=0):
+        return torch.from_numpy(np.random.default_rng(seed).integers(0, vocab, size=(R, L), dtype=np.int64)).to(device)
+
+    def paged(name, workload, P, D, Tb, pool_blocks, save_b, load_b, tok, hash_block):
+        row_bytes = D * 2
+        pool = torch.empty((P, pool_blocks * Tb, D), dtype=torch.int16, device=device)
+        pool.random_(-32768, 32767)
+        table = torch.tensor([pool[p].data_ptr() for p in range(P)], dtype=torch.int64, device=device)
+        B = len(save_b)
+        staging = torch.empty((B, P, Tb, D), dtype=torch.int16, device=device)
+        slots = torch.arange(B, dtype=torch.int32, device=device)
+        d_save, d_load = torch.from_numpy(save_b * Tb).to(device), torch.from_numpy(load_b * Tb).to(device)
+        nbytes = 2 * B * P * Tb * row_bytes
+        ms_g = gpu_ms(torch, lambda: bgs.paged_gather_kv_caches(table, staging, d_save, slots, Tb, D, Tb), reps)
+        ms_s = gpu_ms(torch, lambda: bgs.paged_scatter_kv_caches(table, staging, d_load, slots, Tb, D, Tb), reps)
+        ok = True
+        for b in (0, B // 2, B - 1):
+            s0, l0 = int(save_b[b]) * Tb, int(load_b[b]) * Tb
+            ok &= bool(torch.equal(staging[b], pool[:, s0:s0 + Tb])) and bool(torch.equal(staging[b], pool[:, l0:l0 + Tb]))
+        _, hf = hash_figures(torch, hashing, tok, hash_block, 10)
+        out[name] = dict({"workload": workload, "blocks": B, "tile_bytes": Tb * row_bytes,
+                          "algorithmic_bytes_per_launch": nbytes, "save": copy_figures(ms_g, nbytes),
+                          "load": copy_figures(ms_s, nbytes), "sample_verified": ok}, **hf)
+        del pool, staging
+        release()
+
+    # C1: Qwen2-0.5B-like, 24 layers x K/V, 2 x 64 bf16, 1024-block pool, 128 blocks; 4 x 512 tokens, 256 shared
+    perm = np.random.default_rng(2).permutation(1024).astype(np.int32)
+    tok = np.random.default_rng(0).integers(0, 151936, size=(4, 512), dtype=np.int64)
+    tok[:, :256] = tok[0, :256]
+    paged("C1", "Qwen2-0.5B-like: 24 layers x K/V, 2 KV heads x 64, bf16, 16-token blocks, pool of 1024 blocks, 128 "
+          "blocks moved (2 x 24 MiB per launch: launch-latency bound); 4 requests x 512 tokens hashed",
+          48, 128, 16, 1024, perm[:128], perm[128:256], torch.from_numpy(tok).to(device), 16)
+
+    # C3: 72B-class, 80 layers x K/V, 8 x 128 bf16, 64-token blocks, 8192-block pool; the 25 % missed blocks of
+    # 32 requests x 16384 tokens (2048 blocks, 40 GiB staged)
+    perm = np.random.default_rng(2).permutation(8192).astype(np.int32)
+    miss = np.concatenate([perm[r * 256 + 192:(r + 1) * 256] for r in range(32)])
+    hits = np.concatenate([perm[r * 256:r * 256 + 64] for r in range(32)])
+    paged("C3", "72B-class long context: 80 layers x K/V, 8 KV heads x 128, bf16, 64-token blocks, pool of 8192 blocks; "
+          "the 2048 missed blocks of 32 requests x 16384 tokens (75 % prefix hits) loaded from 40 GiB of staging "
+          "(load is the direction the configuration asks for; save of as many blocks beside it); 32 x 16384 tokens "
+          "hashed in 64-token blocks", 160, 1024, 64, 8192, hits, miss, tokens_uniform(32, 16384, 152064), 64)
+
+    # C4: MLA latent cache in fp8 with one fp32 scale per (layer, block) interleaved into the staged record
+    L4, T4, row4, nblk4 = 61, 128, 576, 4096
+    rec = T4 * row4 + 4
+    pool = torch.empty((L4, nblk4 * T4, row4), dtype=torch.uint8, device=device)
+    pool.random_(0, 126)  # finite e4m3 codes
+    scales = torch.randn((L4, nblk4), dtype=torch.float32, device=device)
+    table = torch.tensor([pool[l].data_ptr() for l in range(L4)], dtype=torch.int64, device=device)
+    ttable = torch.tensor([scales[l].data_ptr() for l in range(L4)], dtype=torch.int64, device=device)
+    blocks = np.random.default_rng(2).permutation(nblk4).astype(np.int32)
+    d_blocks = torch.from_numpy(blocks).to(device)
+    runs = d_blocks * T4
+    staging = torch.empty((nblk4, L4 * rec), dtype=torch.uint8, device=device)
+    desc = _lib.CopyDesc()
+    desc.d_ptr_table, desc.P, desc.ptrs_per_entry, desc.entry_stride_bytes = table.data_ptr(), L4, 1, 0
+    desc.d_staging, desc.staging_block_stride_bytes, desc.staging_tile_stride_bytes = staging.data_ptr(), L4 * rec, rec
+    desc.d_run_start, desc.d_staging_idx, desc.B, desc.T, desc.run_tokens = runs.data_ptr(), None, nblk4, T4, T4
+    desc.slot_limit, desc.row_bytes = 0, row4
+    desc.d_trailer_ptr_table, desc.d_trailer_idx, desc.trailer_bytes = ttable.data_ptr(), d_blocks.data_ptr(), 4
+    desc.max_workgroups = 0
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def launch(fn):
+        rc = fn(desc, stream)
+        if rc != 0:
+            raise SystemExit(f"bench.py: copy with trailers failed with code {rc}")
+
+    nbytes = 2 * nblk4 * L4 * rec
+    ms_g = gpu_ms(torch, lambda: launch(_lib.lib().kvcm_hip_gather_ex), reps)
+    ms_s = gpu_ms(torch, lambda: launch(_lib.lib().kvcm_hip_scatter_ex), reps)  # a full permutation: writes every row back
+    st = staging.view(nblk4, L4, rec)
+    ok = True
+    for b in (0, nblk4 // 2, nblk4 - 1):
+        s0 = int(blocks[b]) * T4
+        ok &= bool(torch.equal(st[b, :, :T4 * row4], pool[:, s0:s0 + T4].reshape(L4, T4 * row4)))
+        ok &= bool(torch.equal(st[b, :, T4 * row4:].contiguous().view(torch.float32).reshape(-1), scales[:, int(blocks[b])]))
+    _, hf = hash_figures(torch, hashing, tokens_uniform(128, 8192, 129280), 128, 10)
+    out["C4"] = dict({"workload": "DeepSeek-V3-style MLA latent cache: 61 layers, 576 e4m3 bytes per token, 128-token "
+                                  "blocks, pool of 4096 blocks, one fp32 scale per (layer, block) interleaved behind "
+                                  "every 73 728-byte tile (records only 4-byte aligned); one full permutation of the "
+                                  "pool (4096 blocks) saved and loaded; 128 requests x 8192 tokens hashed in 128-token "
+                                  "blocks", "blocks": nblk4, "tile_bytes": rec, "algorithmic_bytes_per_launch": nbytes,
+                      "save": copy_figures(ms_g, nbytes), "load": copy_figures(ms_s, nbytes), "sample_verified": ok}, **hf)
+    del pool, staging, scales
+    release()
+
+    # C5: page size 1 (token-granular radix-style paging), 28 layers x K/V, 4 x 128 fp16; 1 048 576 random slots of a
+    # 2 M-slot pool <-> 65 536 storage blocks of 16 tokens; keys of 1024 requests with Zipf-distributed shared prefixes
+    P5, D5, n_slots, B5 = 56, 512, 2 * 1024 * 1024, 65536
+    pool = torch.empty((P5, n_slots, D5), dtype=torch.int16, device=device)
+    pool.random_(-32768, 32767)
+    table = torch.tensor([pool[p].data_ptr() for p in range(P5)], dtype=torch.int64, device=device)
+    perm = np.random.default_rng(2).permutation(n_slots).astype(np.int32)
+    idx_g, idx_s = torch.from_numpy(perm[:B5 * 16]).to(device), torch.from_numpy(perm[B5 * 16:]).to(device)
+    staging = torch.empty((B5, P5, 16, D5), dtype=torch.int16, device=device)
+    slots = torch.arange(B5, dtype=torch.int32, device=device)
+    nbytes = 2 * B5 * P5 * 16 * D5 * 2
+    ms_g = gpu_ms(torch, lambda: bgs.batch_gather_kv_caches(table, staging, idx_g, slots, 16, D5), reps)
+    ms_s = gpu_ms(torch, lambda: bgs.batch_scatter_kv_caches(table, staging, idx_s, slots, 16, D5), reps)
+    ok = True
+    for b in (0, B5 // 2, B5 - 1):
+        gi, si = idx_g[b * 16:(b + 1) * 16].long(), idx_s[b * 16:(b + 1) * 16].long()
+        ok &= bool(torch.equal(staging[b], pool[:, gi])) and bool(torch.equal(staging[b], pool[:, si]))
+    tok5, _, _ = zipf_prefix_tokens(np)
+    keys5, hf = hash_figures(torch, hashing, torch.from_numpy(tok5).to(device), 16, 10)
+    ms_sel = gpu_ms(torch, lambda: save_selection.select_save_indices(keys5), 10)
+    _, count = save_selection.select_save_indices(keys5)
+    out["C5"] = dict({"workload": "page size 1 (Qwen2.5-7B layout: 28 layers x K/V, 4 KV heads x 128, fp16): 1 048 576 "
+                                  "randomly scattered token slots of a 2 M-slot pool <-> 65 536 storage blocks of 16 tokens "
+                                  "(token-granular index, 1 KiB rows); keys of 1024 requests x 1024 tokens with "
+                                  "Zipf(1.2)-distributed shared prefixes, then first occurrences -> save list on the "
+                                  "device", "blocks": B5, "tile_bytes": 16 * D5 * 2, "algorithmic_bytes_per_launch": nbytes,
+                      "save": copy_figures(ms_g, nbytes), "load": copy_figures(ms_s, nbytes), "sample_verified": ok,
+                      "dedup_ms": round(ms_sel, 4), "unique_keys": int(count.item())}, **hf)
+    del pool, staging
+    release()
+    return out
+
+
+def cpu_baseline(np, O, threads, host_cores):
     """The CPU path timed on this host: one memcpy per contiguous chunk between a host-resident pool and
     block-major staging (what the reference's storage SDKs do per Iov), and GenKeyVector per request."""
     P, D = LAYERS * 2, KV_HEADS * HEAD_DIM
@@ -97,25 +303,36 @@ def cpu_baseline(np, O, cores):
         cpu_seconds[0] += spent
         return best
 
-    O.gather_ex(dg, threads=cores)  # warm
+    O.gather_ex(dg, threads=threads)  # warm
     g1 = timed(lambda: O.gather_ex(dg), 2.5)
     s1 = timed(lambda: O.scatter_ex(ds), 2.5)
-    gn = timed(lambda: O.gather_ex(dg, threads=cores), 2.5)
-    sn = timed(lambda: O.scatter_ex(ds, threads=cores), 2.5)
+    gn = timed(lambda: O.gather_ex(dg, threads=threads), 2.5)
+    sn = timed(lambda: O.scatter_ex(ds, threads=threads), 2.5)
+    del pools, staging
 
     rng = np.random.default_rng(0)
     tok = rng.integers(0, VOCAB, size=(REQUESTS, TOKENS_PER_REQ), dtype=np.int64)
     nkeys = REQUESTS * (TOKENS_PER_REQ // T)
-    h1 = timed(lambda: O.hash_tokens(tok, T), 1.5)
-    hn = timed(lambda: O.hash_tokens(tok, T, threads=cores), 1.5)
+    h1 = timed(lambda: O.hash_tokens(tok, T), 1.0)
+    hn = timed(lambda: O.hash_tokens(tok, T, threads=threads), 1.0)
+    # one request per core is only a fair figure on a job that outlasts the start of the threads: 4096 requests of
+    # the same shape (128 MiB of tokens), the 64-request batch 64 times over
+    big_R = 4096
+    big = rng.integers(0, VOCAB, size=(big_R, TOKENS_PER_REQ), dtype=np.int64)
+    big_keys = big_R * (TOKENS_PER_REQ // T)
+    hb = timed(lambda: O.hash_tokens(big, T, threads=threads), 1.5)
     out = {
-        "value": round(2 * moved / (gn + sn) / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+        "value": round(2 * moved / (gn + sn) / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+        "host_cores": host_cores, "threads": threads,
+        "thread_cap": "16 = the CPU share of one GPU on these hosts, whatever the core count of the machine",
         "sample": (f"save+load of {B} blocks (2 GiB staged) between a 4 GiB host pool at the same layout and host "
-                   f"staging, one memcpy per 32 KiB (layer,K/V,block) chunk, {cores} threads; 64x4096-token hash batch; "
-                   f"best of the repetitions that fit 2.5 s (copies) or 1.5 s (hash) per leg"),
+                   f"staging, one memcpy per 32 KiB (layer,K/V,block) chunk, {threads} threads; hash: the 64x4096-token "
+                   f"batch on 1 thread and on {threads}, and {big_R} requests of 4096 tokens on {threads} threads; best of "
+                   f"the repetitions that fit 2.5 s (copies) or 1-1.5 s (hash) per leg"),
         "save_GBps_1thr": round(moved / g1 / 1e9, 2), "load_GBps_1thr": round(moved / s1 / 1e9, 2),
         "save_GBps": round(moved / gn / 1e9, 2), "load_GBps": round(moved / sn / 1e9, 2),
         "hash_keys_per_s_1thr": round(nkeys / h1), "hash_keys_per_s": round(nkeys / hn),
+        "hash_keys_per_s_4096_requests": round(big_keys / hb),
     }
     ref = O.ref()
     if ref is not None:  # the reference's own header, compiled where it lay (oracle/_ref), one request after another
@@ -124,7 +341,7 @@ def cpu_baseline(np, O, cores):
         koff = np.arange(REQUESTS + 1, dtype=np.int64) * (TOKENS_PER_REQ // T)
         keys = np.zeros(nkeys, dtype=np.int64)
         hr = timed(lambda: ref.kvcm_refsrc_hash_tokens(flat.ctypes.data, toff.ctypes.data, REQUESTS, T,
-                                                      keys.ctypes.data, koff.ctypes.data), 1.5)
+                                                      keys.ctypes.data, koff.ctypes.data), 1.0)
         out["hash_keys_per_s_reference_1thr"] = round(nkeys / hr)
     out["cpu_seconds"] = round(cpu_seconds[0], 1)
     return out
@@ -137,6 +354,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--pool-blocks", type=int, default=32768, help="blocks per layer in the paged pool")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="skip configurations 1, 3, 4 and 5")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--calibrate-copy-gib", type=float, default=0.0,
                     help="also run one plain device-to-device copy of this many GiB after the timed region, so that a "
@@ -227,7 +445,60 @@ def main():
         if not ok:
             raise SystemExit("bench.py: results differ from the oracle; refusing to report a number")
 
-    # hash throughput with many chains in flight: 256 batches of the same shape = 16 384 requests (512 MiB of tokens)
+    # ---- the reference-signature call: what data_transfer.py:139-146,206-213 issues per transfer task. Indices are
+    # Python lists of B*T token slots and B staging slots; list -> tensor -> device is inside the timed region. Calls are
+    # issued back to back (the connector keeps 32 of them in flight from its thread pool); `latency` is one call plus
+    # the wait for its completion.
+    task_tok = (inp["save_blocks"][:TASK_BLOCKS, None].astype(np.int64) * T + np.arange(T)[None, :]).reshape(-1).tolist()
+    task_tok_load = (inp["load_blocks"][:TASK_BLOCKS, None].astype(np.int64) * T + np.arange(T)[None, :]).reshape(-1).tolist()
+    task_slots = list(range(TASK_BLOCKS))
+    task_bytes = 2 * TASK_BLOCKS * P * T * row_bytes
+
+    def wall_us(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps * 1e6
+
+    def one_and_wait(fn):
+        def f():
+            fn()
+            torch.cuda.synchronize()
+        return f
+
+    ref_gather = lambda: bgs.batch_gather_kv_caches(inp["ptr_table"], staging, task_tok, task_slots, T, D)
+    ref_scatter = lambda: bgs.batch_scatter_kv_caches(inp["ptr_table"], staging, task_tok_load, task_slots, T, D)
+    d_task_runs = d_save_runs[:TASK_BLOCKS].contiguous()
+    d_task_slots = d_slots[:TASK_BLOCKS].contiguous()
+    fast_gather = lambda: bgs.paged_gather_kv_caches(inp["ptr_table"], staging, d_task_runs, d_task_slots, T, D, T)
+    us_ref_g, us_ref_s = wall_us(ref_gather, 50), wall_us(ref_scatter, 50)
+    reference_signature = {
+        "call": "batch_gather_kv_caches / batch_scatter_kv_caches(ptrs, staging, List[int] of 2048 token slots, "
+                "List[int] of 128 staging slots, 16, 1024): one transfer task, index upload inside the timed region",
+        "blocks_per_task": TASK_BLOCKS, "bytes_per_task": task_bytes,
+        "save_us_per_task": round(us_ref_g, 1), "save_GBps": round(task_bytes / us_ref_g / 1e3, 1),
+        "load_us_per_task": round(us_ref_s, 1), "load_GBps": round(task_bytes / us_ref_s / 1e3, 1),
+        "save_latency_us": round(wall_us(one_and_wait(ref_gather), 20), 1),
+        "load_latency_us": round(wall_us(one_and_wait(ref_scatter), 20), 1),
+        "save_us_per_task_device_block_table": round(wall_us(fast_gather, 50), 1),
+        "save_kernel_us": round(gpu_ms(torch, fast_gather, 50) * 1e3, 1),
+    }
+
+    # ---- the copy kernel on ONE contiguous buffer of the same size (one array, identity block table): what this chip
+    # gives a read+write stream, the ceiling the random-block figures are to be read against
+    flat_src = inp["pool"].view(torch.int16).reshape(-1)[:unique * P * T * D].view(1, unique * P * T, D)
+    flat_table = torch.tensor([flat_src.data_ptr()], dtype=torch.int64, device=device)
+    ident = torch.arange(unique, dtype=torch.int32, device=device) * (P * T)
+    ms_flat = gpu_ms(torch, lambda: bgs.paged_gather_kv_caches(flat_table, staging.view(unique, 1, P * T, D), ident,
+                                                               d_slots, P * T, D, P * T), 5)
+    del flat_src
+    contiguous = copy_figures(ms_flat, copy_bytes)
+
+    # ---- the block-key kernel at other chain counts
+    # 256 batches of the same shape = 16 384 requests (512 MiB of tokens): the HBM-bound regime
     sat_R = 16384
     g = torch.Generator(device=device)
     g.manual_seed(5)
@@ -235,48 +506,54 @@ def main():
     sat_keys = torch.empty(sat_R * (TOKENS_PER_REQ // T), dtype=torch.int64, device=device)
     sat_toff = torch.arange(sat_R + 1, dtype=torch.int64, device=device) * TOKENS_PER_REQ
     sat_koff = torch.arange(sat_R + 1, dtype=torch.int64, device=device) * (TOKENS_PER_REQ // T)
-    hashing.hash_tokens(sat_tokens, T, token_offsets=sat_toff, keys=sat_keys, key_offsets=sat_koff)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(3):
-        hashing.hash_tokens(sat_tokens, T, token_offsets=sat_toff, keys=sat_keys, key_offsets=sat_koff)
-    e1.record()
-    torch.cuda.synchronize()
-    ms_sat = e0.elapsed_time(e1) / 3
+    ms_sat = gpu_ms(torch, lambda: hashing.hash_tokens(sat_tokens, T, token_offsets=sat_toff, keys=sat_keys,
+                                                       key_offsets=sat_koff), 3, warm=1)
     sat_keys_per_s = sat_keys.numel() / (ms_sat * 1e-3)
     sat_alg_bytes = sat_R * TOKENS_PER_REQ * 8 + (sat_R + 1) * 8 * 2 + sat_keys.numel() * 8
-    # ... and with four batches of the configuration hashed in one launch (256 chains): the smallest launch that is
-    # past 1e9 keys/s, since one batch alone is bound by the latency of its 4096 dependent steps
+    # four batches of the configuration in one launch (256 chains): the smallest launch that is past 1e9 keys/s, since
+    # one batch alone is bound by the latency of its 4096 dependent steps
     few_R = 4 * REQUESTS
     few_keys = few_R * (TOKENS_PER_REQ // T)
-    e0.record()
-    for _ in range(10):
-        hashing.hash_tokens(sat_tokens[:few_R], T, token_offsets=sat_toff[:few_R + 1], keys=sat_keys[:few_keys],
-                            key_offsets=sat_koff[:few_R + 1])
-    e1.record()
-    torch.cuda.synchronize()
-    few_keys_per_s = few_keys / (e0.elapsed_time(e1) / 10 * 1e-3)
-    # ... and the one batch of the configuration launched ten times back to back: the step's own pair of events also
-    # times the hand-over from the 8 ms load kernel before it
-    e0.record()
-    for _ in range(10):
-        hashing.hash_tokens(d_tokens, T, token_offsets=d_token_off, keys=d_keys, key_offsets=d_key_off)
-    e1.record()
-    torch.cuda.synchronize()
-    ms_hash_b2b = e0.elapsed_time(e1) / 10
+    ms_few = gpu_ms(torch, lambda: hashing.hash_tokens(sat_tokens[:few_R], T, token_offsets=sat_toff[:few_R + 1],
+                                                       keys=sat_keys[:few_keys], key_offsets=sat_koff[:few_R + 1]), 10)
+    # the one batch of the configuration launched back to back: the step's own pair of events also times the
+    # hand-over from the 8 ms load kernel before it
+    ms_hash_b2b = gpu_ms(torch, lambda: hashing.hash_tokens(d_tokens, T, token_offsets=d_token_off, keys=d_keys,
+                                                            key_offsets=d_key_off), 10)
     del sat_tokens, sat_keys
+
+    digest = kernel_sources_digest()
+    traffic_ok = digest == MEASURED_TRAFFIC["sources_sha256"]
+
+    def traffic(which, same_workload):
+        if traffic_ok and same_workload:
+            return MEASURED_TRAFFIC[which], None
+        why = ("the kernel sources differ from the ones the counters were read on" if not traffic_ok
+               else "the counters were read on the default workload")
+        return None, why
 
     def roof(ms, which):
         achieved = copy_bytes / (ms * 1e-3) / 1e9
-        traffic = MEASURED_TRAFFIC[which] if unique == MEASURED_TRAFFIC["unique_blocks"] else None
-        return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic}
+        tr, why = traffic(which, unique == MEASURED_TRAFFIC["unique_blocks"])
+        r = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+             "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": tr}
+        if why:
+            r["traffic_null_because"] = why
+        return r
 
     roof_g, roof_s = roof(ms_gather, "gather"), roof(ms_scatter, "scatter")
     slower_is_gather = ms_gather >= ms_scatter
     dominant = dict(roof_g if slower_is_gather else roof_s,
                     kernel="copy_span_kernel<16, gather>" if slower_is_gather else "copy_span_kernel<16, scatter>",
                     ms_per_launch=round(max(ms_gather, ms_scatter), 4), algorithmic_bytes_per_launch=copy_bytes)
+    sat_traffic, sat_why = traffic("hash_saturated", True)
+    roof_hash = {"bound": "hbm", "achieved": round(sat_alg_bytes / (ms_sat * 1e-3) / 1e9, 1),
+                 "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                 "frac": round(sat_alg_bytes / (ms_sat * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": sat_traffic,
+                 "kernel": "hash_tokens_kernel<long, 8, 16>", "ms_per_launch": round(ms_sat, 4),
+                 "algorithmic_bytes_per_launch": sat_alg_bytes}
+    if sat_why:
+        roof_hash["traffic_null_because"] = sat_why
 
     result = {
         "metric": "KV save/load GB/s (% of HBM peak) + block-keys/s, Llama-3-8B layout, 1 GPU",
@@ -291,28 +568,34 @@ def main():
                    "requests": REQUESTS, "tokens_per_request": TOKENS_PER_REQ, "block_tokens": T},
         "save_GBps": roof_g["achieved"], "save_frac_of_hbm_peak": roof_g["frac"], "save_ms": round(ms_gather, 4),
         "load_GBps": roof_s["achieved"], "load_frac_of_hbm_peak": roof_s["frac"], "load_ms": round(ms_scatter, 4),
+        "contiguous_copy_same_kernel": contiguous,
         "keys_per_s": round(d_keys.numel() / (ms_hash * 1e-3)), "hash_ms": round(ms_hash, 4), "hash_chains": REQUESTS,
         "hash_ms_back_to_back": round(ms_hash_b2b, 4),
-        "keys_per_s_4_batches": round(few_keys_per_s), "hash_chains_4_batches": few_R,
+        "keys_per_s_back_to_back": round(d_keys.numel() / (ms_hash_b2b * 1e-3)),
+        "hash_floor_us": round(TOKENS_PER_REQ * HASH_STEP_FLOOR_NS * 1e-3, 2),
+        "hash_note": "one request is a serial chain of 4096 dependent steps, three dependent VALU instructions each at "
+                     "3.65 ns: 64 chains cannot finish in less than hash_floor_us; more than 1e9 keys/s needs 256 or more "
+                     "chains in flight (keys_per_s_4_batches)",
+        "keys_per_s_4_batches": round(few_keys / (ms_few * 1e-3)), "hash_chains_4_batches": few_R,
+        "hash_ms_4_batches": round(ms_few, 4),
         "keys_per_s_saturated": round(sat_keys_per_s), "hash_chains_saturated": sat_R,
         "hash_saturated_GBps": round(sat_R * TOKENS_PER_REQ * 8.5 / (ms_sat * 1e-3) / 1e9, 1),
         "verified_against_oracle": verified,
         "roofline": dominant,
-        # the block-key kernel at 16 384 chains: tokens + offsets read, keys written; traffic from the same two
-        # rocprofv3 --pmc runs as the copy kernels (512.6 MiB read + 38.4 MiB written)
-        "roofline_hash_saturated": {"bound": "hbm",
-                                    "achieved": round(sat_alg_bytes / (ms_sat * 1e-3) / 1e9, 1),
-                                    "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                                    "frac": round(sat_alg_bytes / (ms_sat * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-                                    "traffic": MEASURED_TRAFFIC["hash_saturated"] if sat_R == 16384 else None,
-                                    "kernel": "hash_tokens_kernel<long, 8, 16>", "ms_per_launch": round(ms_sat, 4),
-                                    "algorithmic_bytes_per_launch": sat_alg_bytes},
+        "roofline_hash_saturated": roof_hash,
         "roofline_save": roof_g, "roofline_load": roof_s,
+        "reference_signature": reference_signature,
+        "kernel_sources_sha256": digest,
     }
+    del staging, inp
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    if not args.no_configs:
+        result["configs"] = other_configs(torch, np, device)
     if not args.no_cpu_baseline:
         from oracle import oracle as O
-        cores = min(os.cpu_count() or 1, 16)
-        result["cpu_baseline"] = cpu_baseline(np, O, cores)
+        host_cores = os.cpu_count() or 1
+        result["cpu_baseline"] = cpu_baseline(np, O, min(host_cores, 16), host_cores)
     print(json.dumps(result))
 
 

@@ -49,7 +49,7 @@ namespace {
 #define KVCM_COPY_GATHER_STORE_POLICY 1
 #endif
 #ifndef KVCM_COPY_SCATTER_STORE_POLICY
-#define KVCM_COPY_SCATTER_STORE_POLICY 0
+#define KVCM_COPY_SCATTER_STORE_POLICY 2
 #endif
 #ifndef KVCM_COPY_NT_STORE
 #define KVCM_COPY_NT_STORE 1
@@ -99,6 +99,7 @@ struct CopyArgs {
     FastDiv div_entry;
     FastDiv div_units;
     int32_t xcd_remap;
+    int32_t staging_on_line_grid;  // staging base, block stride and tile stride are multiples of 128
 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -219,12 +220,21 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
             slot_shared = runs_b[r_shared];
         }
         const void *pool_first = UNI_TILE ? ptr_table[entry_first] : nullptr;
+        // the span that starts a tile also moves the tile's trailer: its table entries are workgroup-uniform too
+        int32_t trailer_idx_first = -1;
+        const void *trailer_base_first = nullptr;
+        if (UNI_TILE && a.trailer_bytes > 0 && cc_first == 0) {
+            trailer_idx_first = trailer_idx[b];
+            trailer_base_first = trailer_table[p_first];
+        }
         const int64_t slot_b = staging_idx ? staging_idx[b] : static_cast<int64_t>(b);
         unsigned char *block = a.staging + slot_b * a.block_stride;
 
         V v[kCPT];
         unsigned char *pp[kCPT];
         unsigned char *sp[kCPT];
+        uint32_t tr_word = 0;             // a 4-byte trailer in flight, and where it goes
+        unsigned char *tr_dst = nullptr;
 #pragma unroll
         for (int u = 0; u < kCPT; ++u) {
             const uint32_t in_span = threadIdx.x + static_cast<uint32_t>(u) * kThreads;
@@ -247,17 +257,26 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
                     pp[u] = pool + slot * a.row_bytes + static_cast<int64_t>(off) * CS;
                     sp[u] = tile + static_cast<int64_t>(cc) * CS;
                 }
-                if (a.trailer_bytes > 0 && cc == 0 && trailer_idx[b] >= 0) {
+                if (a.trailer_bytes > 0 && cc == 0 && (UNI_TILE ? trailer_idx_first : trailer_idx[b]) >= 0) {
                     // the thread that owns a tile's first chunk also moves the tile's trailer (a negative trailer
                     // index means "no trailer for this block": nothing is read or written)
-                    unsigned char *tr = static_cast<unsigned char *>(const_cast<void *>(trailer_table[p])) +
-                                        static_cast<int64_t>(trailer_idx[b]) * a.trailer_bytes;
+                    const int64_t t_idx = UNI_TILE ? trailer_idx_first : trailer_idx[b];
+                    const void *t_base = UNI_TILE ? trailer_base_first : trailer_table[p];
+                    unsigned char *tr = static_cast<unsigned char *>(const_cast<void *>(t_base)) + t_idx * a.trailer_bytes;
                     unsigned char *st = tile + a.tile_payload;
-                    for (int32_t i = 0; i < a.trailer_bytes; ++i) {
-                        if (SCATTER) {
-                            tr[i] = st[i];
-                        } else {
-                            st[i] = tr[i];
+                    if (a.trailer_bytes == 4 && ((reinterpret_cast<uintptr_t>(tr) | reinterpret_cast<uintptr_t>(st)) & 3u) == 0) {
+                        // one fp32 scale per tile: its load goes out here, next to the load of the thread's own chunk,
+                        // and its store follows the chunk's, so the workgroup that holds this thread does not outlive
+                        // its neighbours by a chain of byte-sized round trips to memory
+                        tr_word = load_chunk<4>(SCATTER ? st : tr);
+                        tr_dst = SCATTER ? tr : st;
+                    } else {
+                        for (int32_t i = 0; i < a.trailer_bytes; ++i) {
+                            if (SCATTER) {
+                                tr[i] = st[i];
+                            } else {
+                                st[i] = tr[i];
+                            }
                         }
                     }
                 }
@@ -283,9 +302,20 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
                     // +1.5 to +4.6 % over non-temporal stores at the BASELINE layouts and +13 % for a 128-block task.
                     // With token-granular indices the same bit costs 2.5 %, and on the pool side of a scatter it
                     // gains nothing: those stay non-temporal.
-                    constexpr int kPolicy = SCATTER ? KVCM_COPY_SCATTER_STORE_POLICY
-                                                    : (RUN == kRunPerGroup ? KVCM_COPY_GATHER_STORE_POLICY : 0);
-                    store_chunk16<kPolicy>(SCATTER ? pp[u] : sp[u], v[u]);
+                    // Block-table form (whole tiles move): the staging side of a gather is written through at system
+                    // scope (sc1), measured +1.5 to +4.6 % over non-temporal stores at the BASELINE layouts and +13 % for
+                    // a 128-block task; the pool side of a scatter carries sc1 and nt together (+1.3 to +2.5 %, and a
+                    // 24 MiB launch that fits the caches finishes 45 % sooner). With token-granular indices either bit
+                    // costs 0.5 to 2.5 %: those stores stay non-temporal. Where staging tiles do not start on cache-line
+                    // boundaries (a 4-byte scale behind every tile) a wave's kilobyte begins and ends inside a line, and
+                    // writing partial lines through costs 15 % (5.2 against 6.0 TB/s): non-temporal there as well.
+                    constexpr int kPolicy = RUN != kRunPerGroup ? 0
+                                            : (SCATTER ? KVCM_COPY_SCATTER_STORE_POLICY : KVCM_COPY_GATHER_STORE_POLICY);
+                    if (kPolicy != 0 && !SCATTER && !a.staging_on_line_grid) {
+                        store_chunk16<0>(sp[u], v[u]);
+                    } else {
+                        store_chunk16<kPolicy>(SCATTER ? pp[u] : sp[u], v[u]);
+                    }
                 } else {
                     store_chunk<CS>(SCATTER ? pp[u] : sp[u], v[u]);
                 }
@@ -310,6 +340,9 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
                     store_chunk<CS>(SCATTER ? pp[u] : sp[u], load_chunk<CS>(SCATTER ? sp[u] : pp[u]));
                 }
             }
+        }
+        if (tr_dst) {
+            store_chunk<4>(tr_dst, tr_word);
         }
     }
 }
@@ -431,6 +464,8 @@ int32_t launch_copy(const kvcm_copy_desc *d, bool scatter, hipStream_t stream) {
     }
     const bool uni_tile = a.chunks_per_tile % kSpan == 0;
     const uint32_t g32 = static_cast<uint32_t>(grid);
+    a.staging_on_line_grid = ((reinterpret_cast<uint64_t>(d->d_staging) | static_cast<uint64_t>(a.block_stride) |
+                               static_cast<uint64_t>(a.tile_stride)) & 127u) == 0;
     if (cs == 16 && uni_tile && a.chunks_per_run % kSpan == 0) {
         launch_span<16, true, kRunPerGroup>(a, d, scatter, g32, stream);
     } else if (cs == 16 && uni_tile && kCPT == 1 && a.chunks_per_run % 64 == 0) {

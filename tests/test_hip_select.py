@@ -103,3 +103,48 @@ def test_workspace_is_checked():
     assert L.kvcm_hip_first_occurrence(keys.data_ptr(), 4096, ws.data_ptr(), need, out.data_ptr(), None, None) == 0
     sync()
     assert (out == 0).all()
+
+
+def test_config5_zipf_shared_prefixes_hash_dedup_gather(oracle):
+    """The page-size-1 configuration's key workload at its own sharing pattern and scale: 1024 requests x 1024 tokens
+    whose shared prefixes are Zipf(1.2)-distributed over 16 templates -> 65 536 keys -> first occurrence of every key
+    -> ascending save list -> gather of exactly those storage blocks (token-granular index). Keys, masks and index
+    list are compared with the oracle, the staged rows with the pool rows they name. Exact."""
+    import bench
+    from tair_kvcache_amd import hashing, save_selection
+    from tair_kvcache_amd.kernel import batch_gather_scatter_helper as bgs
+    toks, which, plen = bench.zipf_prefix_tokens(np)
+    assert toks.shape == (1024, 1024) and len(set(which.tolist())) > 4 and plen.min() >= 64 and plen.max() <= 1024
+    print("config5 zipf: hash", flush=True)
+    keys, koff = hashing.hash_tokens(torch.from_numpy(toks).cuda(), 16)
+    first, rep = save_selection.first_occurrence(keys)
+    idx, count = save_selection.select_save_indices(keys)
+    sync()
+    w_keys, _ = oracle.hash_tokens(toks, 16)
+    assert (keys.cpu().numpy() == w_keys).all()
+    w_first, w_rep = oracle.first_occurrence(w_keys)
+    assert (first.cpu().numpy() == w_first).all() and (rep.cpu().numpy().astype(np.uint8) == w_rep).all()
+    want_idx = oracle.mask_to_indices(w_rep)
+    n = int(count.item())
+    assert n == len(want_idx) and (idx[:n].cpu().numpy() == want_idx).all()
+    # what the sharing pattern implies, derived from the generator's own draws and not from any hash: a block is new
+    # unless an earlier request uses the same template at least that far
+    expect_new = 0
+    longest = {}
+    for r in range(1024):
+        t, blocks = int(which[r]), int(plen[r]) // 16
+        expect_new += 64 - min(blocks, longest.get(t, 0))
+        longest[t] = max(longest.get(t, 0), blocks)
+    assert n == expect_new and n < 65536
+    # gather the blocks to save: storage block k of the batch = 16 token slots of a 2^20-slot pool (4 arrays, 1 KiB rows)
+    P, D, n_slots = 4, 512, 1 << 20
+    pool = torch.randint(-32768, 32767, (P, n_slots, D), dtype=torch.int16, device="cuda")
+    table = torch.tensor([pool[p].data_ptr() for p in range(P)], dtype=torch.int64, device="cuda")
+    slot_of_token = torch.from_numpy(np.random.default_rng(2).permutation(n_slots).astype(np.int32)).cuda()
+    tidx = slot_of_token.view(65536, 16)[idx[:n].long()].contiguous()      # [n, 16] token slots of the blocks to save
+    staging = torch.zeros((n, P, 16, D), dtype=torch.int16, device="cuda")
+    print(f"config5 zipf: gather {n} of 65536 blocks", flush=True)
+    bgs.batch_gather_kv_caches(table, staging, tidx, torch.arange(n, dtype=torch.int32, device="cuda"), 16, D)
+    sync()
+    for p in range(P):
+        assert torch.equal(staging[:, p].reshape(n * 16, D), pool[p][tidx.reshape(-1).long()]), p
