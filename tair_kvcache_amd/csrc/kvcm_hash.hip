@@ -12,7 +12,7 @@
 //               after its producer and independent ones 1.75 ns apart (measured), so the step is written for
 //               depth: three dependent levels, 5 instructions (see chain_step).
 //   waves 1..3  "loader waves": stream the 64 requests' tokens from HBM in [64 requests x 64 tokens] tiles with
-//               16-byte buffer loads (512-byte row segments), add C, and write them transposed into a 3-slot LDS
+//               16-byte buffer loads (512-byte row segments), add C, and write them transposed into a 2-slot LDS
 //               ring. Each loader wave owns every third tile and keeps its loads in flight for about three
 //               tile periods, so HBM latency stays off the chain.
 // Roofline: HBM for many requests (8*block_size + 8 bytes per key); for few requests the bound is the
@@ -39,9 +39,16 @@ constexpr int kLoaders = KVCM_HASH_LOADERS;
 constexpr int kThreads = 64 * (1 + kLoaders);
 constexpr int kReqs = 64;                     // requests per workgroup = lanes of the chain wave
 constexpr int kTT = KVCM_HASH_TILE_TOKENS;    // tokens per request per tile
-constexpr int kRing = 3;                      // LDS tiles in the ring: computed on, prefetched from, written to
+constexpr int kRing = 2;                      // LDS tiles in the ring: prefetched from, written to (the tile that is
+                                              // computed on already sits in the chain wave's registers)
 constexpr int kPad = 2;                       // keeps rows 16-byte aligned (b128 reads) and spreads banks
 constexpr int kPerLane = kReqs * kTT / 64;  // tile elements per loader lane
+// Staged keys (many requests in flight, block size 16): the keys of kKeyGroupTiles tiles collect in LDS and leave as
+// whole rows of 512 bytes per request, see hash_tokens_kernel.
+constexpr int kKeyGroupTiles = 16;
+constexpr int kKeysPerGroup = kKeyGroupTiles * (kTT / 16);
+constexpr int kKeyPad = 2;
+constexpr int kKeyRow = kKeysPerGroup + kKeyPad;  // one request's row of the LDS key buffer
 
 // Workgroup barrier that waits only for this wave's LDS traffic. __syncthreads() would also drain the
 // loader waves' outstanding global loads, which must stay in flight across barriers.
@@ -192,10 +199,40 @@ struct GlobalLoader {
 // which the chain wave pulled into registers an iteration ago). A loader issues the loads of its next tile right
 // AFTER the barrier that published its previous one, so they stay in flight for kLoaders - 1 tile periods while the
 // data waits in the loader's registers, not in LDS: more loaders = more bytes in flight per CU at no LDS cost.
-template <typename Loader, typename TokT>
+// What a loader wave needs to write out a group of staged keys (KS kernels only).
+struct KeyDrain {
+    const uint64_t *s_keys;   // LDS: [2][request][kKeyRow] keys of the group being filled and of the one before
+    const int64_t *s_keypos;                                    // LDS: index of each request's first key, -1 = no request
+    int64_t *keys;
+    int32_t full_tiles;  // tiles in which no request has run out of tokens
+};
+
+// One group of staged keys, LDS -> global: every store instruction writes two requests' rows of 512 bytes, whole cache
+// lines, non-temporal. Written as 8-byte stores from the chain wave (one line per lane, a sixteenth of it at a time)
+// the 32 MiB of keys of a 16 384-request batch cost 20 us of a 107 us launch -- not for their bytes but for what they do
+// to the memory system in the middle of the token stream; the same stores into a buffer that stays in the L2 cost
+// nothing, and so do they as one burst after the last token. Whole rows at intervals of sixteen tiles recover a third
+// of that.
+__device__ __forceinline__ void drain_keys(const KeyDrain &kd, int32_t group, uint32_t lane) {
+    const uint32_t buf = static_cast<uint32_t>(group) & 1u;
+#pragma unroll 8
+    for (int j = 0; j < kReqs * kKeysPerGroup / 128; ++j) {
+        const uint32_t c = static_cast<uint32_t>(j) * 64u + lane;  // 16-byte piece of the group's keys
+        const uint32_t row = c / (kKeysPerGroup / 2), piece = c % (kKeysPerGroup / 2);
+        const int64_t first = kd.s_keypos[row];
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(kd.s_keys + (buf * kReqs + row) * kKeyRow + piece * 2);
+        if (first >= 0) {
+            typedef u32x4 u32x4_a8 __attribute__((aligned(8)));
+            __builtin_nontemporal_store(
+                v, reinterpret_cast<u32x4_a8 *>(kd.keys + first + static_cast<int64_t>(group) * kKeysPerGroup + piece * 2));
+        }
+    }
+}
+
+template <typename Loader, typename TokT, bool KS>
 __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t (*s_tile)[kReqs][kTT + kPad],
-                                           int64_t lw, int64_t ntiles, uint32_t lane) {
-    static_assert(kRing == 3 && kLoaders >= 3, "three ring slots: computed on, prefetched from, written to");
+                                           int64_t lw, int64_t ntiles, uint32_t lane, const KeyDrain &kd) {
+    static_assert(kRing == 2 && kLoaders >= 3, "two ring slots: prefetched from, written to");
     Loader ld;
     ld.setup(ctx, lane);
     // 32-bit counters: the loop control stays in scalar registers (there are no ordered 64-bit scalar compares); a
@@ -211,12 +248,15 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
     if (me < 2 && me + kLoaders < nt) {
         ld.issue(static_cast<int64_t>(me + kLoaders) * kTT);
     }
+    // tile 2 goes where tile 0 lies: not before the chain wave has pulled tile 0 into its registers
+    lds_barrier();
     int32_t turn = 2 % kLoaders;  // loader whose tile is due: (k + 2) % kLoaders
-    int slot = 2;                 // ring slot of that tile: (k + 2) % kRing
+    int slot = 2 % kRing;         // ring slot of that tile: (k + 2) % kRing
     bool was_mine = false;
     for (int32_t k = 0; k < nt; ++k) {
         const int32_t nxt = k + 2;  // tile that must be in LDS when this iteration ends
-        const bool mine = turn == me && nxt < nt;
+        const bool my_turn = turn == me;
+        const bool mine = my_turn && nxt < nt;
         if (mine) {
             ld.store(s_tile[slot]);
         }
@@ -232,6 +272,13 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
             ld.template issue_half<1>(static_cast<int64_t>(nxt - 1 + kLoaders) * kTT);
         }
         was_mine = mine;
+        if (KS && (k & (kKeyGroupTiles - 1)) == kKeyGroupTiles - 1 && k < kd.full_tiles) {
+            // the barrier above closed a group of staged keys. The loader that has just published a tile writes them
+            // out: its next wait for memory is three tiles away, so the stores are not waited for
+            if (my_turn) {
+                drain_keys(kd, k / kKeyGroupTiles, lane);
+            }
+        }
     }
 }
 
@@ -243,10 +290,13 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
 // BS > 0 = the block size is this compile-time constant (a divisor or a multiple of the tile): the places where a key
 // is due are then known when the code is written, and the scalar bookkeeping (add, compare, branch per chunk: one
 // instruction slot in sixteen of the wave that sets the pace) disappears from the loop.
-template <int CHUNK, bool MASKED, int BS>
+// STAGED (unmasked tiles, block size 16): the tile's keys go to the lane's row of the LDS key buffer, `staged_row`
+// pointing at the tile's first key there; a loader wave writes the rows out (drain_keys).
+template <int CHUNK, bool MASKED, int BS, bool STAGED = false>
 __device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_t &h, int64_t t0, int64_t my_ntok,
                                          int32_t &since_key, int32_t block_size, int64_t *__restrict__ keys,
-                                         int64_t &key_pos) {
+                                         int64_t &key_pos, uint64_t *staged_row = nullptr) {
+    static_assert(!STAGED || (!MASKED && BS == 16), "keys are staged for whole tiles of 16-token blocks only");
     static_assert(BS == 0 || (BS % CHUNK == 0 && (kTT % BS == 0 || BS % kTT == 0)), "block size fits the tiling");
     // tokens of this lane that are hashed and lie in this tile or before its end: a block that ends at position p of
     // the tile belongs to the lane iff p <= left (my_ntok is a multiple of the block size)
@@ -271,7 +321,9 @@ __device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_
             key_due = c + CHUNK == kTT && (t0 + kTT) % BS == 0;
         }
         if (key_due) {
-            if (!MASKED || c + CHUNK <= left) {
+            if (STAGED) {
+                staged_row[(c + CHUNK) / (BS > 0 ? BS : 1) - 1] = h;
+            } else if (!MASKED || c + CHUNK <= left) {
                 keys[key_pos] = static_cast<int64_t>(h);
             }
             key_pos += 1;
@@ -289,7 +341,10 @@ __device__ __forceinline__ void read_row(ulonglong2 (&a)[kTT / 2], const uint64_
 
 // CHUNK = steps between two looks at the block boundary: 8 when block_size % 8 == 0 (a lane is then
 // active for whole chunks or not at all), otherwise 1. BS = block size when it is 1, 8, 16, 32, 64 or 128, otherwise 0.
-template <typename TokT, int CHUNK, int BS>
+// KS ("keys staged", block size 16 only; chosen by the host for batches of many requests, where the launch is bound by
+// memory and not by the chain): the chain wave writes its keys into an LDS buffer instead of to memory, and after every
+// kKeyGroupTiles tiles in which every request is whole a loader wave writes the group out as rows of 512 bytes.
+template <typename TokT, int CHUNK, int BS, bool KS = false>
 __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__restrict__ tokens,
                                                               const int64_t *__restrict__ token_offsets, int32_t R,
                                                               int32_t block_size, uint64_t seed,
@@ -299,6 +354,9 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     __shared__ __attribute__((aligned(16))) uint64_t s_tile[kRing][kReqs][kTT + kPad];
     __shared__ int64_t s_start[kReqs];
     __shared__ int64_t s_ntok[kReqs];
+    static_assert(!KS || BS == 16, "keys are staged for 16-token blocks");
+    __shared__ __attribute__((aligned(16))) uint64_t s_keys[KS ? 2 * kReqs * kKeyRow : 2];
+    __shared__ int64_t s_keypos[KS ? kReqs : 1];
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -319,6 +377,9 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         }
         s_start[lane] = start;
         s_ntok[lane] = my_ntok;
+        if (KS) {
+            s_keypos[lane] = r < R ? key_pos : -1;
+        }
     } else {
         ctx.tokens = tokens;
         ctx.s_start = s_start;
@@ -354,12 +415,16 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         return;
     }
 
+    // tiles [0, n_full) are those in which no request has run out of tokens
+    const int64_t full = min_ntok / kTT;
+    const int32_t n_full = static_cast<int32_t>(full < ntiles ? full : ntiles);
     if (wave != 0) {
         // ---------------------------------------------------------------- loader waves
+        const KeyDrain kd{s_keys, s_keypos, keys, n_full};
         if (buffer_loads) {
-            run_loader<BufferLoader<TokT>, TokT>(ctx, s_tile, wave - 1, ntiles, lane);
+            run_loader<BufferLoader<TokT>, TokT, KS>(ctx, s_tile, wave - 1, ntiles, lane, kd);
         } else {
-            run_loader<GlobalLoader<TokT>, TokT>(ctx, s_tile, wave - 1, ntiles, lane);
+            run_loader<GlobalLoader<TokT>, TokT, KS>(ctx, s_tile, wave - 1, ntiles, lane, kd);
         }
         return;
     }
@@ -376,12 +441,10 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     }
     ulonglong2 cur[kTT / 2], nxt[kTT / 2];
     read_row(cur, &s_tile[0][lane][0]);
+    lds_barrier();  // tile 0 is in registers: its slot may take tile 2
     // Loop control in 32-bit scalars (there are no ordered 64-bit scalar compares, and every vector compare is an issue
-    // slot of this wave): tiles [0, n_full) are those in which no lane has run out of tokens. A request of 2^37 tokens
-    // does not fit the memory of the device, so the tile count fits 32 bits.
+    // slot of this wave). A request of 2^37 tokens does not fit the memory of the device, so the tile count fits 32 bits.
     const int32_t nt = static_cast<int32_t>(ntiles);
-    const int64_t full = min_ntok / kTT;
-    const int32_t n_full = static_cast<int32_t>(full < ntiles ? full : ntiles);
     int ring = 0;
     for (int32_t k = 0; k < nt; k += 2) {
         // even tile: compute on `cur`, prefetch the odd tile into `nxt`; then the other way round
@@ -389,7 +452,16 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         if (k + 1 < nt) {
             read_row(nxt, &s_tile[ring1][lane][0]);
         }
-        if (k < n_full) {
+        // a group of kKeyGroupTiles tiles is staged when all of its tiles are whole for every request; k and k + 1 lie
+        // in the same group
+        const int32_t group = k / kKeyGroupTiles;
+        const bool staged = KS && (group + 1) * kKeyGroupTiles <= n_full;
+        uint64_t *staged_row = KS ? s_keys + ((group & 1) * kReqs + lane) * kKeyRow + (k & (kKeyGroupTiles - 1)) * (kTT / 16)
+                                  : nullptr;
+        if (KS && staged) {
+            run_tile<CHUNK, false, BS, KS>(cur, h, static_cast<int64_t>(k) * kTT, my_ntok, since_key, block_size, keys,
+                                           key_pos, staged_row);
+        } else if (k < n_full) {
             run_tile<CHUNK, false, BS>(cur, h, static_cast<int64_t>(k) * kTT, my_ntok, since_key, block_size, keys,
                                        key_pos);
         } else {
@@ -404,7 +476,10 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         if (k + 2 < nt) {
             read_row(cur, &s_tile[ring][lane][0]);
         }
-        if (k + 1 < n_full) {
+        if (KS && staged) {
+            run_tile<CHUNK, false, BS, KS>(nxt, h, static_cast<int64_t>(k + 1) * kTT, my_ntok, since_key, block_size,
+                                           keys, key_pos, staged_row + kTT / 16);
+        } else if (k + 1 < n_full) {
             run_tile<CHUNK, false, BS>(nxt, h, static_cast<int64_t>(k + 1) * kTT, my_ntok, since_key, block_size, keys,
                                        key_pos);
         } else {
@@ -552,6 +627,12 @@ std::atomic<int32_t> g_force_global_loads{[] {
     return (fg && fg[0] == '1') ? 1 : 0;
 }()};
 
+// From this many requests in one launch the keys of 16-token blocks are staged in LDS (hash_tokens_kernel<.., KS>).
+#ifndef KVCM_HASH_STAGED_FROM
+#define KVCM_HASH_STAGED_FROM 8192
+#endif
+constexpr int32_t kStagedKeysFromRequests = KVCM_HASH_STAGED_FROM;
+
 template <typename TokT>
 int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_t R, int32_t block_size, int64_t seed,
                     int64_t *d_keys, const int64_t *d_key_offsets, hipStream_t stream) {
@@ -569,7 +650,12 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
 #define KVCM_LAUNCH_HASH(CHUNK, BS)                                                                                  \
     hipLaunchKernelGGL((hash_tokens_kernel<TokT, CHUNK, BS>), grid, dim3(kThreads), 0, stream, d_tokens,            \
                        d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
-    if (block_size == 16) {  // the engines' usual block sizes get kernels of their own
+    if (block_size == 16 && R >= kStagedKeysFromRequests) {
+        // many chains in flight: memory sets the pace, and how the keys are written is a fifth of the launch
+        hipLaunchKernelGGL((hash_tokens_kernel<TokT, 8, 16, true>), grid, dim3(kThreads), 0, stream, d_tokens,
+                           d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets,
+                           force_global);
+    } else if (block_size == 16) {  // the engines' usual block sizes get kernels of their own
         KVCM_LAUNCH_HASH(8, 16);
     } else if (block_size == 8) {
         KVCM_LAUNCH_HASH(8, 8);

@@ -159,3 +159,33 @@ def test_bad_buffers_are_refused_on_the_host():
     keys, _ = h.hash_tokens(flat, 16, token_offsets=off)                                     # and the good call works
     sync()
     assert keys.numel() == 16
+
+
+@pytest.mark.parametrize("dtype", [np.int64, np.int32])
+@pytest.mark.parametrize("shape", ["uniform", "uniform_odd_count", "ragged", "ragged_short", "two_lengths"])
+def test_many_requests_take_the_staged_key_path(oracle, dtype, shape):
+    """From 8192 requests in one launch the keys of 16-token blocks are collected in LDS and written out as 512-byte
+    rows by a loader wave; groups of tiles in which some request has run out, requests past a multiple of 64, and
+    whatever does not fill a group of sixteen tiles go the direct way. Every mixture against the oracle, exact."""
+    rng = np.random.default_rng(5)
+    lens = {
+        "uniform": np.full(8192, 2048),                                # two whole groups per request
+        "uniform_odd_count": np.full(8192 + 37, 1024 + 64 * 3 + 5),    # one group + three tiles + a tail; last workgroup partial
+        "ragged": rng.integers(1100, 3000, size=8300),                 # first group whole for everyone, later ones not
+        "ragged_short": rng.integers(0, 1500, size=9000),              # many workgroups with no whole group at all
+        "two_lengths": np.where(np.arange(8192) % 64 < 32, 4096, 2048),  # half of every workgroup ends after two groups
+    }[shape].astype(np.int64)
+    toff = np.zeros(len(lens) + 1, dtype=np.int64)
+    np.cumsum(lens, out=toff[1:])
+    if dtype == np.int32:
+        flat = rng.integers(-2**31, 2**31 - 1, size=int(toff[-1]), dtype=np.int64).astype(np.int32)
+    else:
+        flat = rng.integers(-2**63, 2**63 - 1, size=int(toff[-1]), dtype=np.int64)
+    print(f"staged keys case {shape} {np.dtype(dtype).name}: {len(lens)} requests, {int(toff[-1])} tokens", flush=True)
+    want, woff = oracle.hash_tokens(flat, 16, token_offsets=toff, seed=3, threads=8)
+    keys = torch.full((len(want) + 64,), -7, dtype=torch.int64, device="cuda")    # room behind the keys: must stay untouched
+    d_koff = dev(woff)
+    got, off = _h().hash_tokens(dev(flat), 16, token_offsets=dev(toff), seed=3, keys=keys, key_offsets=d_koff)
+    sync()
+    assert (host(got, np.int64)[:len(want)] == want).all()
+    assert (host(got, np.int64)[len(want):] == -7).all()
