@@ -87,6 +87,29 @@ __device__ __forceinline__ uint64_t pre_add_i32(uint32_t token) {
     return sum;
 }
 
+// Maximum / minimum of a 32-bit value over the 64 lanes of a wave, returned as a wave-uniform value. Data-parallel
+// primitives within rows of 16 lanes, then across rows: six steps of one or two instructions, against six round trips
+// through the LDS crossbar for the shuffle form (0.5 us at the head of a kernel that lasts 50).
+template <bool MAX>
+__device__ __forceinline__ uint32_t wave_reduce_u32(uint32_t v) {
+#define KVCM_DPP_STEP(CTRL)                                                                                       \
+    {                                                                                                             \
+        const uint32_t o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(static_cast<int>(v), static_cast<int>(v), \
+                                                                             CTRL, 0xf, 0xf, false));             \
+        v = MAX ? (o > v ? o : v) : (o < v ? o : v);                                                              \
+    }
+    KVCM_DPP_STEP(0x111)  // row_shr:1   a lane without a source keeps its own value
+    KVCM_DPP_STEP(0x112)  // row_shr:2
+    KVCM_DPP_STEP(0x114)  // row_shr:4
+    KVCM_DPP_STEP(0x118)  // row_shr:8   lane 15 of every row now holds the row's result
+    KVCM_DPP_STEP(0x142)  // row_bcast:15
+    KVCM_DPP_STEP(0x143)  // row_bcast:31  lane 63 holds the wave's
+#undef KVCM_DPP_STEP
+    return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), 63));
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) { return wave_reduce_u32<true>(v); }
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) { return wave_reduce_u32<false>(v); }
+
 // What a loader wave needs to know about its workgroup.
 template <typename TokT>
 struct LoaderCtx {
@@ -395,29 +418,18 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     }
     __syncthreads();
 
-    // min over the requests that exist: the rows past R of the last workgroup do not make it "ragged"
-    int64_t max_ntok = s_ntok[lane];
-    int64_t min_ntok = r < R ? max_ntok : INT64_MAX;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const int64_t hi_other = __shfl_xor(max_ntok, o);
-        const int64_t lo_other = __shfl_xor(min_ntok, o);
-        max_ntok = hi_other > max_ntok ? hi_other : max_ntok;
-        min_ntok = lo_other < min_ntok ? lo_other : min_ntok;
-    }
-    // the reductions left the same value in every lane; say so, and loop control becomes scalar
-    max_ntok = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(max_ntok >> 32))) << 32) |
-               __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(max_ntok));
-    min_ntok = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(min_ntok >> 32))) << 32) |
-               __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(min_ntok));
-    const int64_t ntiles = (max_ntok + kTT - 1) / kTT;  // uniform over the workgroup
+    // Tiles of the longest request (how long the workgroup runs) and whole tiles of the shortest (from where on some
+    // lane has run out): max and min over the 64 lanes of per-lane tile counts, which fit 32 bits (a request of 2^37
+    // tokens does not fit the memory of the device). Rows past R in the last workgroup count for neither.
+    const int64_t lane_ntok = s_ntok[lane];
+    const uint32_t ntiles_u = wave_max_u32(static_cast<uint32_t>((lane_ntok + kTT - 1) / kTT));
+    const uint32_t full_u = wave_min_u32(r < R ? static_cast<uint32_t>(lane_ntok / kTT) : 0xFFFFFFFFu);
+    const int64_t ntiles = ntiles_u;  // uniform over the workgroup
     if (ntiles == 0) {
         return;
     }
-
     // tiles [0, n_full) are those in which no request has run out of tokens
-    const int64_t full = min_ntok / kTT;
-    const int32_t n_full = static_cast<int32_t>(full < ntiles ? full : ntiles);
+    const int32_t n_full = static_cast<int32_t>(full_u < ntiles_u ? full_u : ntiles_u);
     if (wave != 0) {
         // ---------------------------------------------------------------- loader waves
         const KeyDrain kd{s_keys, s_keypos, keys, n_full};
