@@ -236,11 +236,15 @@ struct KeyDrain {
 // to the memory system in the middle of the token stream; the same stores into a buffer that stays in the L2 cost
 // nothing, and so do they as one burst after the last token. Whole rows at intervals of sixteen tiles recover a third
 // of that.
-__device__ __forceinline__ void drain_keys(const KeyDrain &kd, int32_t group, uint32_t lane) {
+// A group is 32 such store instructions; `step` (0..15) selects two of them, so that the work spreads over the sixteen
+// tiles that follow the group instead of holding one loader back from its next barrier.
+constexpr int kDrainSteps = kKeyGroupTiles;
+constexpr int kDrainPerStep = kReqs * kKeysPerGroup / 128 / kDrainSteps;
+__device__ __forceinline__ void drain_keys(const KeyDrain &kd, int32_t group, int32_t step, uint32_t lane) {
     const uint32_t buf = static_cast<uint32_t>(group) & 1u;
-#pragma unroll 8
-    for (int j = 0; j < kReqs * kKeysPerGroup / 128; ++j) {
-        const uint32_t c = static_cast<uint32_t>(j) * 64u + lane;  // 16-byte piece of the group's keys
+#pragma unroll
+    for (int j = 0; j < kDrainPerStep; ++j) {
+        const uint32_t c = static_cast<uint32_t>(step * kDrainPerStep + j) * 64u + lane;  // 16-byte piece of the group's keys
         const uint32_t row = c / (kKeysPerGroup / 2), piece = c % (kKeysPerGroup / 2);
         const int64_t first = kd.s_keypos[row];
         const u32x4 v = *reinterpret_cast<const u32x4 *>(kd.s_keys + (buf * kReqs + row) * kKeyRow + piece * 2);
@@ -283,6 +287,14 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
         if (mine) {
             ld.store(s_tile[slot]);
         }
+        if (KS && k >= kKeyGroupTiles && (k / kKeyGroupTiles) * kKeyGroupTiles <= kd.full_tiles &&
+            (turn == 0 ? kLoaders - 1 : turn - 1) == me) {
+            // The group of staged keys before the one this tile belongs to was closed by an earlier barrier, and its
+            // buffer is not written again before the barrier that ends this group: a sixteenth of it leaves per tile,
+            // here, in front of the barrier, through the loader that published a tile an iteration ago and has nothing
+            // to do until the barrier (its own next wait for memory is two tiles away, so the stores are not waited for).
+            drain_keys(kd, k / kKeyGroupTiles - 1, k & (kKeyGroupTiles - 1), lane);
+        }
         turn = turn + 1 == kLoaders ? 0 : turn + 1;
         slot = slot + 1 == kRing ? 0 : slot + 1;
         lds_barrier();
@@ -295,11 +307,17 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
             ld.template issue_half<1>(static_cast<int64_t>(nxt - 1 + kLoaders) * kTT);
         }
         was_mine = mine;
-        if (KS && (k & (kKeyGroupTiles - 1)) == kKeyGroupTiles - 1 && k < kd.full_tiles) {
-            // the barrier above closed a group of staged keys. The loader that has just published a tile writes them
-            // out: its next wait for memory is three tiles away, so the stores are not waited for
-            if (my_turn) {
-                drain_keys(kd, k / kKeyGroupTiles, lane);
+    }
+    if (KS) {
+        // What the loop did not reach of the last staged group (all of it when the request ends with the group), the
+        // steps dealt out to the loaders; no barrier follows, and nobody writes the buffers any more.
+        const int32_t last = kd.full_tiles / kKeyGroupTiles - 1;
+        if (last >= 0) {
+            const int32_t done = nt - (last + 1) * kKeyGroupTiles;  // steps the loop has taken for this group
+            for (int32_t step = done < 0 ? 0 : done; step < kDrainSteps; ++step) {
+                if (step % kLoaders == me) {
+                    drain_keys(kd, last, step, lane);
+                }
             }
         }
     }
@@ -644,6 +662,11 @@ std::atomic<int32_t> g_force_global_loads{[] {
 #define KVCM_HASH_STAGED_FROM 8192
 #endif
 constexpr int32_t kStagedKeysFromRequests = KVCM_HASH_STAGED_FROM;
+// ... and, for 8-byte tokens, only below this many (one workgroup of 64 requests per CU of an MI355X).
+#ifndef KVCM_HASH_STAGED_UNTIL_8
+#define KVCM_HASH_STAGED_UNTIL_8 (64 * 256)
+#endif
+constexpr int32_t kStagedKeysUntilRequests8 = KVCM_HASH_STAGED_UNTIL_8;
 
 template <typename TokT>
 int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_t R, int32_t block_size, int64_t seed,
@@ -662,8 +685,12 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
 #define KVCM_LAUNCH_HASH(CHUNK, BS)                                                                                  \
     hipLaunchKernelGGL((hash_tokens_kernel<TokT, CHUNK, BS>), grid, dim3(kThreads), 0, stream, d_tokens,            \
                        d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
-    if (block_size == 16 && R >= kStagedKeysFromRequests) {
-        // many chains in flight: memory sets the pace, and how the keys are written is a fifth of the launch
+    // Staged keys pay where the launch is not bound by the token stream alone: 4-byte tokens (16 384 requests: 58 us
+    // against 68), or 8-byte tokens with fewer workgroups than the 256 CUs (8192 requests: 65 us against 72.5). With
+    // 8-byte tokens and a workgroup on every CU the staged form is 2 % slower (108 us against 106), so it stays out.
+    const bool staged_keys = block_size == 16 && R >= kStagedKeysFromRequests &&
+                             (sizeof(TokT) == 4 || R < kStagedKeysUntilRequests8);
+    if (staged_keys) {
         hipLaunchKernelGGL((hash_tokens_kernel<TokT, 8, 16, true>), grid, dim3(kThreads), 0, stream, d_tokens,
                            d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets,
                            force_global);
