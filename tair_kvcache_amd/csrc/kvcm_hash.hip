@@ -256,7 +256,47 @@ __device__ __forceinline__ void drain_keys(const KeyDrain &kd, int32_t group, in
     }
 }
 
-template <typename Loader, typename TokT, bool KS>
+// Half of a closed group (`part` = 0 or 1: every other store instruction), in bursts of eight row pieces: all LDS reads
+// of a burst are under way before its first store goes out, so the loader is back at its loads after about 0.2 us.
+__device__ __forceinline__ void drain_half(const KeyDrain &kd, int32_t group, int32_t part, uint32_t lane) {
+    const uint32_t buf = static_cast<uint32_t>(group) & 1u;
+    constexpr int kBurst = 8;
+    static_assert((kDrainSteps * kDrainPerStep / 2) % kBurst == 0, "whole bursts");
+    typedef u32x4 u32x4_a8 __attribute__((aligned(8)));
+#pragma unroll 1
+    for (int32_t base = 0; base < kDrainSteps * kDrainPerStep / 2; base += kBurst) {
+        int64_t first[kBurst];
+        u32x4 v[kBurst];
+        uint32_t piece[kBurst];
+#pragma unroll
+        for (int i = 0; i < kBurst; ++i) {
+            const uint32_t c = static_cast<uint32_t>((base + i) * 2 + part) * 64u + lane;
+            const uint32_t row = c / (kKeysPerGroup / 2);
+            piece[i] = c % (kKeysPerGroup / 2);
+            first[i] = kd.s_keypos[row];
+            v[i] = *reinterpret_cast<const u32x4 *>(kd.s_keys + (buf * kReqs + row) * kKeyRow + piece[i] * 2);
+        }
+#pragma unroll
+        for (int i = 0; i < kBurst; ++i) {
+            if (first[i] >= 0) {
+                __builtin_nontemporal_store(
+                    v[i], reinterpret_cast<u32x4_a8 *>(kd.keys + first[i] + static_cast<int64_t>(group) * kKeysPerGroup +
+                                                      piece[i] * 2));
+            }
+        }
+    }
+}
+
+// How a kernel's keys reach memory: from the chain wave, one at a time (kKeysDirect); staged in LDS and written by the
+// loaders a sixteenth of a group per tile (kKeysSpread); staged and written a whole group at once, right after the
+// barrier that closes it (kKeysBurst). Measured on 4096-token requests, us per launch, direct / spread / burst:
+// 16 384 requests of 8-byte tokens 106 / 107 / 102, 65 536 requests of 1024 8-byte tokens 111 / 107 / 104,
+// 8192 requests 72 / 65 / 66, 16 384 requests of 4-byte tokens 68 / 59 / 65. Writes that all workgroups issue at the
+// same moments disturb the token stream less than writes spread evenly through it, as long as the loaders do not fall
+// behind while they issue them.
+constexpr int kKeysDirect = 0, kKeysSpread = 1, kKeysBurst = 2;
+
+template <typename Loader, typename TokT, int KS>
 __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t (*s_tile)[kReqs][kTT + kPad],
                                            int64_t lw, int64_t ntiles, uint32_t lane, const KeyDrain &kd) {
     static_assert(kRing == 2 && kLoaders >= 3, "two ring slots: prefetched from, written to");
@@ -287,7 +327,7 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
         if (mine) {
             ld.store(s_tile[slot]);
         }
-        if (KS && k >= kKeyGroupTiles && (k / kKeyGroupTiles) * kKeyGroupTiles <= kd.full_tiles &&
+        if (KS == kKeysSpread && k >= kKeyGroupTiles && (k / kKeyGroupTiles) * kKeyGroupTiles <= kd.full_tiles &&
             (turn == 0 ? kLoaders - 1 : turn - 1) == me) {
             // The group of staged keys before the one this tile belongs to was closed by an earlier barrier, and its
             // buffer is not written again before the barrier that ends this group: a sixteenth of it leaves per tile,
@@ -307,8 +347,13 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
             ld.template issue_half<1>(static_cast<int64_t>(nxt - 1 + kLoaders) * kTT);
         }
         was_mine = mine;
+        if (KS == kKeysBurst && (k & (kKeyGroupTiles - 1)) == kKeyGroupTiles - 1 && k < kd.full_tiles && turn != me) {
+            // The barrier above closed a group. The loader whose tile is due next leaves it alone (its next wait for
+            // memory would wait for these stores as well); the other two write half of it each.
+            drain_half(kd, k / kKeyGroupTiles, (me - turn + kLoaders) % kLoaders - 1, lane);
+        }
     }
-    if (KS) {
+    if (KS == kKeysSpread) {
         // What the loop did not reach of the last staged group (all of it when the request ends with the group), the
         // steps dealt out to the loaders; no barrier follows, and nobody writes the buffers any more.
         const int32_t last = kd.full_tiles / kKeyGroupTiles - 1;
@@ -382,10 +427,11 @@ __device__ __forceinline__ void read_row(ulonglong2 (&a)[kTT / 2], const uint64_
 
 // CHUNK = steps between two looks at the block boundary: 8 when block_size % 8 == 0 (a lane is then
 // active for whole chunks or not at all), otherwise 1. BS = block size when it is 1, 8, 16, 32, 64 or 128, otherwise 0.
-// KS ("keys staged", block size 16 only; chosen by the host for batches of many requests, where the launch is bound by
-// memory and not by the chain): the chain wave writes its keys into an LDS buffer instead of to memory, and after every
-// kKeyGroupTiles tiles in which every request is whole a loader wave writes the group out as rows of 512 bytes.
-template <typename TokT, int CHUNK, int BS, bool KS = false>
+// KS != kKeysDirect ("keys staged", block size 16 only; chosen by the host for batches of many requests, where the launch
+// is bound by memory and not by the chain): the chain wave writes its keys into an LDS buffer instead of to memory, and
+// after every kKeyGroupTiles tiles in which every request is whole the loader waves write the group out as rows of 512
+// bytes, spread over the next group's tiles or at once.
+template <typename TokT, int CHUNK, int BS, int KS = kKeysDirect>
 __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__restrict__ tokens,
                                                               const int64_t *__restrict__ token_offsets, int32_t R,
                                                               int32_t block_size, uint64_t seed,
@@ -489,7 +535,7 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         uint64_t *staged_row = KS ? s_keys + ((group & 1) * kReqs + lane) * kKeyRow + (k & (kKeyGroupTiles - 1)) * (kTT / 16)
                                   : nullptr;
         if (KS && staged) {
-            run_tile<CHUNK, false, BS, KS>(cur, h, static_cast<int64_t>(k) * kTT, my_ntok, since_key, block_size, keys,
+            run_tile<CHUNK, false, BS, KS != kKeysDirect>(cur, h, static_cast<int64_t>(k) * kTT, my_ntok, since_key, block_size, keys,
                                            key_pos, staged_row);
         } else if (k < n_full) {
             run_tile<CHUNK, false, BS>(cur, h, static_cast<int64_t>(k) * kTT, my_ntok, since_key, block_size, keys,
@@ -507,7 +553,7 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
             read_row(cur, &s_tile[ring][lane][0]);
         }
         if (KS && staged) {
-            run_tile<CHUNK, false, BS, KS>(nxt, h, static_cast<int64_t>(k + 1) * kTT, my_ntok, since_key, block_size,
+            run_tile<CHUNK, false, BS, KS != kKeysDirect>(nxt, h, static_cast<int64_t>(k + 1) * kTT, my_ntok, since_key, block_size,
                                            keys, key_pos, staged_row + kTT / 16);
         } else if (k + 1 < n_full) {
             run_tile<CHUNK, false, BS>(nxt, h, static_cast<int64_t>(k + 1) * kTT, my_ntok, since_key, block_size, keys,
@@ -662,11 +708,11 @@ std::atomic<int32_t> g_force_global_loads{[] {
 #define KVCM_HASH_STAGED_FROM 8192
 #endif
 constexpr int32_t kStagedKeysFromRequests = KVCM_HASH_STAGED_FROM;
-// ... and, for 8-byte tokens, only below this many (one workgroup of 64 requests per CU of an MI355X).
-#ifndef KVCM_HASH_STAGED_UNTIL_8
-#define KVCM_HASH_STAGED_UNTIL_8 (64 * 256)
+// ... and, for 8-byte tokens, from this many (one workgroup of 64 requests per CU of an MI355X) a group leaves at once.
+#ifndef KVCM_HASH_BURST_FROM_8
+#define KVCM_HASH_BURST_FROM_8 (64 * 256)
 #endif
-constexpr int32_t kStagedKeysUntilRequests8 = KVCM_HASH_STAGED_UNTIL_8;
+constexpr int32_t kBurstKeysFromRequests8 = KVCM_HASH_BURST_FROM_8;
 
 template <typename TokT>
 int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_t R, int32_t block_size, int64_t seed,
@@ -685,15 +731,17 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
 #define KVCM_LAUNCH_HASH(CHUNK, BS)                                                                                  \
     hipLaunchKernelGGL((hash_tokens_kernel<TokT, CHUNK, BS>), grid, dim3(kThreads), 0, stream, d_tokens,            \
                        d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
-    // Staged keys pay where the launch is not bound by the token stream alone: 4-byte tokens (16 384 requests: 58 us
-    // against 68), or 8-byte tokens with fewer workgroups than the 256 CUs (8192 requests: 65 us against 72.5). With
-    // 8-byte tokens and a workgroup on every CU the staged form is 2 % slower (108 us against 106), so it stays out.
-    const bool staged_keys = block_size == 16 && R >= kStagedKeysFromRequests &&
-                             (sizeof(TokT) == 4 || R < kStagedKeysUntilRequests8);
-    if (staged_keys) {
-        hipLaunchKernelGGL((hash_tokens_kernel<TokT, 8, 16, true>), grid, dim3(kThreads), 0, stream, d_tokens,
-                           d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets,
-                           force_global);
+    // Staged keys pay where the launch is not bound by the chain alone (the figures stand at kKeysDirect): spread over
+    // the tiles for 4-byte tokens and for 8-byte tokens that leave CUs idle, in bursts once every CU has a workgroup.
+    const bool staged_keys = block_size == 16 && R >= kStagedKeysFromRequests;
+    const bool burst = sizeof(TokT) == 8 && R >= kBurstKeysFromRequests8;
+#define KVCM_LAUNCH_HASH_STAGED(KS)                                                                                  \
+    hipLaunchKernelGGL((hash_tokens_kernel<TokT, 8, 16, KS>), grid, dim3(kThreads), 0, stream, d_tokens,            \
+                       d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
+    if (staged_keys && burst) {
+        KVCM_LAUNCH_HASH_STAGED(kKeysBurst);
+    } else if (staged_keys) {
+        KVCM_LAUNCH_HASH_STAGED(kKeysSpread);
     } else if (block_size == 16) {  // the engines' usual block sizes get kernels of their own
         KVCM_LAUNCH_HASH(8, 16);
     } else if (block_size == 8) {
@@ -711,6 +759,7 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
     } else {
         KVCM_LAUNCH_HASH(1, 0);
     }
+#undef KVCM_LAUNCH_HASH_STAGED
 #undef KVCM_LAUNCH_HASH
     return launch_status();
 }

@@ -163,11 +163,13 @@ def test_bad_buffers_are_refused_on_the_host():
 
 @pytest.mark.parametrize("dtype", [np.int64, np.int32])
 @pytest.mark.parametrize("shape", ["uniform", "uniform_odd_count", "ragged", "ragged_short", "two_lengths",
-                                   "workgroup_on_every_cu"])
+                                   "workgroup_on_every_cu", "every_cu_ragged", "every_cu_two_lengths"])
 def test_many_requests_take_the_staged_key_path(oracle, dtype, shape):
-    """From 8192 requests in one launch (8-byte tokens: up to 16 383) the keys of 16-token blocks are collected in LDS
-    and written out as 512-byte rows by the loader waves, a sixteenth of a group per tile and the rest after the loop; groups of tiles in which some request has run out, requests past a multiple of 64, and
-    whatever does not fill a group of sixteen tiles go the direct way. Every mixture against the oracle, exact."""
+    """From 8192 requests in one launch the keys of 16-token blocks are collected in LDS and written out as 512-byte
+    rows by the loader waves: a sixteenth of a group per tile and the rest after the loop, or (8-byte tokens, from
+    16 384 requests) a whole group right after the barrier that closes it. Groups of tiles in which some request has run
+    out, requests past a multiple of 64, and whatever does not fill a group of sixteen tiles go the direct way. Every
+    mixture against the oracle, exact."""
     rng = np.random.default_rng(5)
     lens = {
         "uniform": np.full(8192, 2048),                                # two whole groups per request
@@ -175,7 +177,9 @@ def test_many_requests_take_the_staged_key_path(oracle, dtype, shape):
         "ragged": rng.integers(1100, 3000, size=8300),                 # first group whole for everyone, later ones not
         "ragged_short": rng.integers(0, 1500, size=9000),              # many workgroups with no whole group at all
         "two_lengths": np.where(np.arange(8192) % 64 < 32, 4096, 2048),  # half of every workgroup ends after two groups
-        "workgroup_on_every_cu": np.full(16384 + 70, 1024 + 100),      # from 16 384 requests only 4-byte tokens are staged
+        "workgroup_on_every_cu": np.full(16384 + 70, 1024 + 100),      # one group + a tile + a tail; last workgroup partial
+        "every_cu_ragged": rng.integers(1100, 3000, size=16384 + 70),
+        "every_cu_two_lengths": np.where(np.arange(16384) % 64 < 32, 3072, 1024),
     }[shape].astype(np.int64)
     toff = np.zeros(len(lens) + 1, dtype=np.int64)
     np.cumsum(lens, out=toff[1:])
