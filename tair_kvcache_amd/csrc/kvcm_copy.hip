@@ -26,7 +26,9 @@
 //   registers; nothing is reshaped in memory. When a span lies inside one tile (and one run) the tile number,
 //   pool pointer and slot are workgroup-uniform: scalar arithmetic and scalar loads, and a thread's own work is
 //   two address adds. Otherwise chunk -> (tile, run, offset) is two multiply-shift divisions per thread.
-//   All accesses carry the non-temporal hint: every byte is touched once (+4 % gather against plain accesses).
+//   Every byte is touched once: loads carry the non-temporal hint (+4 % gather against plain accesses), and so
+//   do stores, except where whole tiles move (block-table form): there the staging side of a gather is written
+//   through at system scope and the pool side of a scatter carries both bits (see the store site below).
 //
 // Roofline: HBM. Algorithmic bytes per tile = 2 * T * row_bytes (+ trailer), index bytes are negligible.
 #include "kvcm_internal.h"
@@ -298,10 +300,6 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
 #pragma unroll
             for (int u = 0; u < kCPT; ++u) {
                 if constexpr (CS == 16) {
-                    // Staging written in whole tiles (block-table form): written through at system scope, measured
-                    // +1.5 to +4.6 % over non-temporal stores at the BASELINE layouts and +13 % for a 128-block task.
-                    // With token-granular indices the same bit costs 2.5 %, and on the pool side of a scatter it
-                    // gains nothing: those stay non-temporal.
                     // Block-table form (whole tiles move): the staging side of a gather is written through at system
                     // scope (sc1), measured +1.5 to +4.6 % over non-temporal stores at the BASELINE layouts and +13 % for
                     // a 128-block task; the pool side of a scatter carries sc1 and nt together (+1.3 to +2.5 %, and a

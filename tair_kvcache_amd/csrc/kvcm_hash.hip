@@ -14,7 +14,9 @@
 //   waves 1..3  "loader waves": stream the 64 requests' tokens from HBM in [64 requests x 64 tokens] tiles with
 //               16-byte buffer loads (512-byte row segments), add C, and write them transposed into a 2-slot LDS
 //               ring. Each loader wave owns every third tile and keeps its loads in flight for about three
-//               tile periods, so HBM latency stays off the chain.
+//               tile periods, so HBM latency stays off the chain. In launches of thousands of requests they also
+//               write the keys out: the chain wave leaves them in an LDS buffer, and whole 512-byte rows per
+//               request go to memory (kKeysSpread / kKeysBurst) instead of one 8-byte store per key and lane.
 // Roofline: HBM for many requests (8*block_size + 8 bytes per key); for few requests the bound is the
 // dependent-instruction latency of the chain wave, which no amount of bandwidth removes.
 #include "kvcm_internal.h"

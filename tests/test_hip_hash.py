@@ -195,3 +195,21 @@ def test_many_requests_take_the_staged_key_path(oracle, dtype, shape):
     sync()
     assert (host(got, np.int64)[:len(want)] == want).all()
     assert (host(got, np.int64)[len(want):] == -7).all()
+
+
+@pytest.mark.parametrize("dtype,R", [(np.int64, 16384 + 70), (np.int64, 8300), (np.int32, 8300)])
+def test_staged_keys_with_the_general_loader(oracle, force_general_hash_loader, dtype, R):
+    """The staged-key forms (spread and burst) are loader code as well: both with the loader that a workgroup spanning
+    4 GiB of tokens would take, ragged requests, exact."""
+    force_general_hash_loader(True)
+    rng = np.random.default_rng(23)
+    lens = rng.integers(1030, 2300, size=R).astype(np.int64)
+    toff = np.zeros(R + 1, dtype=np.int64)
+    np.cumsum(lens, out=toff[1:])
+    flat = rng.integers(-2**31, 2**31 - 1, size=int(toff[-1]), dtype=np.int64).astype(dtype)
+    print(f"staged keys, general loader: {R} requests of {np.dtype(dtype).name}, {int(toff[-1])} tokens", flush=True)
+    want, woff = oracle.hash_tokens(flat, 16, token_offsets=toff, threads=8)
+    keys, off = _h().hash_tokens(dev(flat), 16, token_offsets=dev(toff))
+    sync()
+    assert (host(keys, np.int64) == want).all()
+
