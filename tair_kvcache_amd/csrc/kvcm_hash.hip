@@ -157,10 +157,13 @@ struct BufferLoader {
         const uint32_t tile_off = static_cast<uint32_t>(t0 * sizeof(TokT));
 #pragma unroll
         for (int j = HALF * (kNL / 2); j < (HALF + 1) * (kNL / 2); ++j) {
-            // aux = 2: the non-temporal bit. Tokens are read once; with 8-byte tokens the bit is worth 17 % at
-            // 16 384 requests (107 us against 125 us), with 4-byte tokens it COSTS 10 % (83 us against 75 us),
-            // measured with sc0, sc1 and both as well: only nt matters.
-            regs[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, rel[j] + tile_off, 0, sizeof(TokT) == 8 ? 2 : 0);
+            // aux = 2: the non-temporal bit (sc0, sc1 and both were measured as well: only nt matters). Tokens are
+            // read once. Timed the way the kernel is used -- on tokens that are not in the 256 MiB memory-side cache,
+            // which holds other dirty data -- the bit is worth 30 to 45 % from 4096 requests up, for either token
+            // width (8192 x 4096 8-byte tokens: 68 us against 96; 16 384 x 4096 4-byte tokens: 83 against 125) and
+            // 5 % for one batch. Launched over and over on the same 256 MiB or less, the kernel without the bit reads
+            // that cache instead of HBM and looks 10 to 25 % faster than with it: a benchmark's artefact.
+            regs[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, rel[j] + tile_off, 0, 2);
         }
     }
     // Adds the golden-ratio constant (the token term of the step is v + C) and writes the tile transposed.
@@ -264,7 +267,6 @@ __device__ __forceinline__ void drain_half(const KeyDrain &kd, int32_t group, in
     const uint32_t buf = static_cast<uint32_t>(group) & 1u;
     constexpr int kBurst = 8;
     static_assert((kDrainSteps * kDrainPerStep / 2) % kBurst == 0, "whole bursts");
-    typedef u32x4 u32x4_a8 __attribute__((aligned(8)));
 #pragma unroll 1
     for (int32_t base = 0; base < kDrainSteps * kDrainPerStep / 2; base += kBurst) {
         int64_t first[kBurst];
@@ -281,9 +283,10 @@ __device__ __forceinline__ void drain_half(const KeyDrain &kd, int32_t group, in
 #pragma unroll
         for (int i = 0; i < kBurst; ++i) {
             if (first[i] >= 0) {
-                __builtin_nontemporal_store(
-                    v[i], reinterpret_cast<u32x4_a8 *>(kd.keys + first[i] + static_cast<int64_t>(group) * kKeysPerGroup +
-                                                      piece[i] * 2));
+                // written through at system scope: 97-99 us for 16 384 x 4096 tokens where the same stores take
+                // 101-105 us non-temporal, 104 plain, 100-101 with sc1 alone (65 536 x 4096: 385-388 against 399-403 us)
+                int64_t *dst = kd.keys + first[i] + static_cast<int64_t>(group) * kKeysPerGroup + piece[i] * 2;
+                asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" : : "v"(dst), "v"(v[i]) : "memory");
             }
         }
     }
@@ -291,11 +294,9 @@ __device__ __forceinline__ void drain_half(const KeyDrain &kd, int32_t group, in
 
 // How a kernel's keys reach memory: from the chain wave, one at a time (kKeysDirect); staged in LDS and written by the
 // loaders a sixteenth of a group per tile (kKeysSpread); staged and written a whole group at once, right after the
-// barrier that closes it (kKeysBurst). Measured on 4096-token requests, us per launch, direct / spread / burst:
-// 16 384 requests of 8-byte tokens 106 / 107 / 102, 65 536 requests of 1024 8-byte tokens 111 / 107 / 104,
-// 8192 requests 72 / 65 / 66, 16 384 requests of 4-byte tokens 68 / 59 / 65. Writes that all workgroups issue at the
-// same moments disturb the token stream less than writes spread evenly through it, as long as the loaders do not fall
-// behind while they issue them.
+// barrier that closes it (kKeysBurst); the host chooses by token width and number of requests (the timings stand at
+// launch_hash). Writes that all workgroups issue at the same moments disturb the token stream less than writes spread
+// evenly through it, as long as the loaders do not fall behind while they issue them.
 constexpr int kKeysDirect = 0, kKeysSpread = 1, kKeysBurst = 2;
 
 template <typename Loader, typename TokT, int KS>
@@ -705,16 +706,23 @@ std::atomic<int32_t> g_force_global_loads{[] {
     return (fg && fg[0] == '1') ? 1 : 0;
 }()};
 
-// From this many requests in one launch the keys of 16-token blocks are staged in LDS (hash_tokens_kernel<.., KS>).
-#ifndef KVCM_HASH_STAGED_FROM
-#define KVCM_HASH_STAGED_FROM 8192
+// From how many requests in one launch the keys of 16-token blocks are staged in LDS and written by the loader waves
+// (hash_tokens_kernel<.., KS>), spread over the tiles or a group at a time. Chosen from timings on tokens that are not
+// in the memory-side cache, us for requests of 4096 tokens, direct / spread / burst:
+//   8-byte tokens   1024: 61 / 59 / 63    4096: 65 / 61 / 64     8192: 76 / 68 / 70      10 240: 83 / 76 / 73
+//                   12 288: 92 / 85 / 83  16 384: 112 / 111 / 107    32 768: 227 / 219 / 209
+//   4-byte tokens   4096: 56 / 58 / 63    8192: 58 / 58 / 64     10 240: 64 / 62 / 66    12 288: 72 / 66 / 67
+//                   16 384: 85 / 81 / 78  32 768: 159 / 151 / 151
+// (4-byte tokens never take the spread form: two of the three are enough code.)
+#ifndef KVCM_HASH_SPREAD_FROM_8
+#define KVCM_HASH_SPREAD_FROM_8 4096
 #endif
-constexpr int32_t kStagedKeysFromRequests = KVCM_HASH_STAGED_FROM;
-// ... and, for 8-byte tokens, from this many (one workgroup of 64 requests per CU of an MI355X) a group leaves at once.
 #ifndef KVCM_HASH_BURST_FROM_8
-#define KVCM_HASH_BURST_FROM_8 (64 * 256)
+#define KVCM_HASH_BURST_FROM_8 10240
 #endif
-constexpr int32_t kBurstKeysFromRequests8 = KVCM_HASH_BURST_FROM_8;
+#ifndef KVCM_HASH_BURST_FROM_4
+#define KVCM_HASH_BURST_FROM_4 12288
+#endif
 
 template <typename TokT>
 int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_t R, int32_t block_size, int64_t seed,
@@ -733,17 +741,18 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
 #define KVCM_LAUNCH_HASH(CHUNK, BS)                                                                                  \
     hipLaunchKernelGGL((hash_tokens_kernel<TokT, CHUNK, BS>), grid, dim3(kThreads), 0, stream, d_tokens,            \
                        d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
-    // Staged keys pay where the launch is not bound by the chain alone (the figures stand at kKeysDirect): spread over
-    // the tiles for 4-byte tokens and for 8-byte tokens that leave CUs idle, in bursts once every CU has a workgroup.
-    const bool staged_keys = block_size == 16 && R >= kStagedKeysFromRequests;
-    const bool burst = sizeof(TokT) == 8 && R >= kBurstKeysFromRequests8;
+    constexpr bool k8 = sizeof(TokT) == 8;
+    const bool burst = block_size == 16 && R >= (k8 ? KVCM_HASH_BURST_FROM_8 : KVCM_HASH_BURST_FROM_4);
+    const bool spread = block_size == 16 && k8 && !burst && R >= KVCM_HASH_SPREAD_FROM_8;
 #define KVCM_LAUNCH_HASH_STAGED(KS)                                                                                  \
     hipLaunchKernelGGL((hash_tokens_kernel<TokT, 8, 16, KS>), grid, dim3(kThreads), 0, stream, d_tokens,            \
                        d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
-    if (staged_keys && burst) {
+    if (burst) {
         KVCM_LAUNCH_HASH_STAGED(kKeysBurst);
-    } else if (staged_keys) {
-        KVCM_LAUNCH_HASH_STAGED(kKeysSpread);
+    } else if (spread) {
+        if constexpr (k8) {
+            KVCM_LAUNCH_HASH_STAGED(kKeysSpread);
+        }
     } else if (block_size == 16) {  // the engines' usual block sizes get kernels of their own
         KVCM_LAUNCH_HASH(8, 16);
     } else if (block_size == 8) {

@@ -165,11 +165,11 @@ def test_bad_buffers_are_refused_on_the_host():
 @pytest.mark.parametrize("shape", ["uniform", "uniform_odd_count", "ragged", "ragged_short", "two_lengths",
                                    "workgroup_on_every_cu", "every_cu_ragged", "every_cu_two_lengths"])
 def test_many_requests_take_the_staged_key_path(oracle, dtype, shape):
-    """From 8192 requests in one launch the keys of 16-token blocks are collected in LDS and written out as 512-byte
-    rows by the loader waves: a sixteenth of a group per tile and the rest after the loop, or (8-byte tokens, from
-    16 384 requests) a whole group right after the barrier that closes it. Groups of tiles in which some request has run
-    out, requests past a multiple of 64, and whatever does not fill a group of sixteen tiles go the direct way. Every
-    mixture against the oracle, exact."""
+    """In launches of thousands of requests the keys of 16-token blocks are collected in LDS and written out as
+    512-byte rows by the loader waves: a sixteenth of a group per tile and the rest after the loop (8-byte tokens, 4096
+    to 10 239 requests), or a whole group right after the barrier that closes it (8-byte tokens from 10 240 requests,
+    4-byte tokens from 12 288). Groups of tiles in which some request has run out, requests past a multiple of 64, and
+    whatever does not fill a group of sixteen tiles go the direct way. Every mixture against the oracle, exact."""
     rng = np.random.default_rng(5)
     lens = {
         "uniform": np.full(8192, 2048),                                # two whole groups per request
@@ -197,7 +197,7 @@ def test_many_requests_take_the_staged_key_path(oracle, dtype, shape):
     assert (host(got, np.int64)[len(want):] == -7).all()
 
 
-@pytest.mark.parametrize("dtype,R", [(np.int64, 16384 + 70), (np.int64, 8300), (np.int32, 8300)])
+@pytest.mark.parametrize("dtype,R", [(np.int64, 16384 + 70), (np.int64, 8300), (np.int32, 12288 + 70)])
 def test_staged_keys_with_the_general_loader(oracle, force_general_hash_loader, dtype, R):
     """The staged-key forms (spread and burst) are loader code as well: both with the loader that a workgroup spanning
     4 GiB of tokens would take, ragged requests, exact."""
