@@ -20,6 +20,7 @@ Prints ONE JSON line. Runs on one GPU only.
 """
 import argparse
 import hashlib
+import itertools
 import json
 import os
 import sys
@@ -37,8 +38,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # were measured on: a run whose sources differ reports traffic null and says why.
 KERNEL_SOURCES = ("tair_kvcache_amd/csrc/kvcm_copy.hip", "tair_kvcache_amd/csrc/kvcm_hash.hip",
                   "tair_kvcache_amd/csrc/kvcm_internal.h")
-MEASURED_TRAFFIC = {"sources_sha256": "2e9ef9307ca40fab", "unique_blocks": 12416, "gather": 52076677486,
-                    "scatter": 52076200785, "hash_saturated": 571047947}
+MEASURED_TRAFFIC = {"sources_sha256": "063b8f4a11f784b5", "unique_blocks": 12416, "gather": 52076669955,
+                    "scatter": 52076195353, "hash_saturated": 571006300}
 
 # Llama-3-8B KV layout: the configuration the headline metric is quoted on
 LAYERS, KV_HEADS, HEAD_DIM, ITEMSIZE = 32, 8, 128, 2
@@ -483,10 +484,18 @@ def main():
     # Python lists of B*T token slots and B staging slots; list -> tensor -> device is inside the timed region. Calls are
     # issued back to back (the connector keeps 32 of them in flight from its thread pool); `latency` is one call plus
     # the wait for its completion.
-    task_tok = (inp["save_blocks"][:TASK_BLOCKS, None].astype(np.int64) * T + np.arange(T)[None, :]).reshape(-1).tolist()
-    task_tok_load = (inp["load_blocks"][:TASK_BLOCKS, None].astype(np.int64) * T + np.arange(T)[None, :]).reshape(-1).tolist()
-    task_slots = list(range(TASK_BLOCKS))
+    # Every call takes the next 128 blocks of the save (load) list and the next 128 staging slots, as the connector's
+    # tasks do: a task that moved the same 512 MiB over and over would be served by the 256 MiB memory-side cache.
+    n_tasks = unique // TASK_BLOCKS
+
+    def task_lists(blocks):
+        return [(blocks[i * TASK_BLOCKS:(i + 1) * TASK_BLOCKS, None].astype(np.int64) * T +
+                 np.arange(T)[None, :]).reshape(-1).tolist() for i in range(n_tasks)]
+
+    task_tok, task_tok_load = task_lists(inp["save_blocks"]), task_lists(inp["load_blocks"])
+    task_slots = [list(range(i * TASK_BLOCKS, (i + 1) * TASK_BLOCKS)) for i in range(n_tasks)]
     task_bytes = 2 * TASK_BLOCKS * P * T * row_bytes
+    turn = itertools.count()
 
     def wall_us(fn, reps):
         fn()
@@ -503,15 +512,26 @@ def main():
             torch.cuda.synchronize()
         return f
 
-    ref_gather = lambda: bgs.batch_gather_kv_caches(inp["ptr_table"], staging, task_tok, task_slots, T, D)
-    ref_scatter = lambda: bgs.batch_scatter_kv_caches(inp["ptr_table"], staging, task_tok_load, task_slots, T, D)
-    d_task_runs = d_save_runs[:TASK_BLOCKS].contiguous()
-    d_task_slots = d_slots[:TASK_BLOCKS].contiguous()
-    fast_gather = lambda: bgs.paged_gather_kv_caches(inp["ptr_table"], staging, d_task_runs, d_task_slots, T, D, T)
+    def ref_gather():
+        i = next(turn) % n_tasks
+        bgs.batch_gather_kv_caches(inp["ptr_table"], staging, task_tok[i], task_slots[i], T, D)
+
+    def ref_scatter():
+        i = next(turn) % n_tasks
+        bgs.batch_scatter_kv_caches(inp["ptr_table"], staging, task_tok_load[i], task_slots[i], T, D)
+
+    d_task_runs = [d_save_runs[i * TASK_BLOCKS:(i + 1) * TASK_BLOCKS].contiguous() for i in range(n_tasks)]
+    d_task_slots = [d_slots[i * TASK_BLOCKS:(i + 1) * TASK_BLOCKS].contiguous() for i in range(n_tasks)]
+
+    def fast_gather():
+        i = next(turn) % n_tasks
+        bgs.paged_gather_kv_caches(inp["ptr_table"], staging, d_task_runs[i], d_task_slots[i], T, D, T)
+
     us_ref_g, us_ref_s = wall_us(ref_gather, 50), wall_us(ref_scatter, 50)
     reference_signature = {
         "call": "batch_gather_kv_caches / batch_scatter_kv_caches(ptrs, staging, List[int] of 2048 token slots, "
-                "List[int] of 128 staging slots, 16, 1024): one transfer task, index upload inside the timed region",
+                "List[int] of 128 staging slots, 16, 1024): one transfer task, index upload inside the timed region; "
+                "every call moves the next 128 of the 12 416 blocks",
         "blocks_per_task": TASK_BLOCKS, "bytes_per_task": task_bytes,
         "save_us_per_task": round(us_ref_g, 1), "save_GBps": round(task_bytes / us_ref_g / 1e3, 1),
         "load_us_per_task": round(us_ref_s, 1), "load_GBps": round(task_bytes / us_ref_s / 1e3, 1),
