@@ -232,7 +232,7 @@ struct KeyDrain {
     const uint64_t *s_keys;   // LDS: [2][request][kKeyRow] keys of the group being filled and of the one before
     const int64_t *s_keypos;                                    // LDS: index of each request's first key, -1 = no request
     int64_t *keys;
-    int32_t full_tiles;  // tiles in which no request has run out of tokens
+    int32_t full_tiles;  // tiles in which no request has run out of tokens and whose keys may be staged
 };
 
 // One group of staged keys, LDS -> global: every store instruction writes two requests' rows of 512 bytes, whole cache
@@ -298,6 +298,43 @@ __device__ __forceinline__ void drain_half(const KeyDrain &kd, int32_t group, in
 // launch_hash). Writes that all workgroups issue at the same moments disturb the token stream less than writes spread
 // evenly through it, as long as the loaders do not fall behind while they issue them.
 constexpr int kKeysDirect = 0, kKeysSpread = 1, kKeysBurst = 2;
+// A workgroup of a spread kernel whose requests are shorter than this many tiles stores its keys directly: what the last
+// group costs after the loop (about 1.5 us) is more than staging saves on 2048 tokens.
+constexpr int kSpreadFromTiles = 32;
+
+// The steps [first_step, kDrainSteps) of a group that belong to loader `me` (step % kLoaders == me), all LDS reads
+// under way before the first store: nothing else is left to do when this runs, so round trips would add up.
+__device__ __forceinline__ void drain_tail(const KeyDrain &kd, int32_t group, int32_t first_step, int32_t me,
+                                           uint32_t lane) {
+    const uint32_t buf = static_cast<uint32_t>(group) & 1u;
+    constexpr int kMaxSteps = (kDrainSteps + kLoaders - 1) / kLoaders;
+    constexpr int kN = kMaxSteps * kDrainPerStep;
+    typedef u32x4 u32x4_a8 __attribute__((aligned(8)));
+    const int32_t s0 = first_step + (me - first_step % kLoaders + kLoaders) % kLoaders;
+    int64_t first[kN];
+    u32x4 v[kN];
+    uint32_t piece[kN];
+#pragma unroll
+    for (int i = 0; i < kN; ++i) {
+        const int32_t step = s0 + (i / kDrainPerStep) * kLoaders;
+        first[i] = -1;
+        if (step < kDrainSteps) {
+            const uint32_t c = static_cast<uint32_t>(step * kDrainPerStep + i % kDrainPerStep) * 64u + lane;
+            const uint32_t row = c / (kKeysPerGroup / 2);
+            piece[i] = c % (kKeysPerGroup / 2);
+            first[i] = kd.s_keypos[row];
+            v[i] = *reinterpret_cast<const u32x4 *>(kd.s_keys + (buf * kReqs + row) * kKeyRow + piece[i] * 2);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kN; ++i) {
+        if (first[i] >= 0) {
+            __builtin_nontemporal_store(
+                v[i], reinterpret_cast<u32x4_a8 *>(kd.keys + first[i] + static_cast<int64_t>(group) * kKeysPerGroup +
+                                                  piece[i] * 2));
+        }
+    }
+}
 
 template <typename Loader, typename TokT, int KS>
 __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t (*s_tile)[kReqs][kTT + kPad],
@@ -343,11 +380,20 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
         lds_barrier();
         // the loads of this loader's next tile go out in two halves, one tile period apart: a burst of 32 load
         // instructions sits in the CU's memory pipeline in front of the chain wave's key stores
-        if (mine && nxt + kLoaders < nt) {
-            ld.template issue_half<0>(static_cast<int64_t>(nxt + kLoaders) * kTT);
-        }
-        if (was_mine && nxt - 1 + kLoaders < nt) {
-            ld.template issue_half<1>(static_cast<int64_t>(nxt - 1 + kLoaders) * kTT);
+        // (which of the two forms runs is a compile-time matter: with both in one loop body the compiler waits for
+        // all outstanding loads where the paths meet, and a kernel that does so takes 80 us for a batch instead of 58)
+        if (KS == kKeysSpread) {
+            // no key stores of the chain wave to keep out of the way of: 2 to 5 % faster from 4096 requests than in halves
+            if (mine && nxt + kLoaders < nt) {
+                ld.issue(static_cast<int64_t>(nxt + kLoaders) * kTT);
+            }
+        } else {
+            if (mine && nxt + kLoaders < nt) {
+                ld.template issue_half<0>(static_cast<int64_t>(nxt + kLoaders) * kTT);
+            }
+            if (was_mine && nxt - 1 + kLoaders < nt) {
+                ld.template issue_half<1>(static_cast<int64_t>(nxt - 1 + kLoaders) * kTT);
+            }
         }
         was_mine = mine;
         if (KS == kKeysBurst && (k & (kKeyGroupTiles - 1)) == kKeyGroupTiles - 1 && k < kd.full_tiles && turn != me) {
@@ -362,11 +408,7 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
         const int32_t last = kd.full_tiles / kKeyGroupTiles - 1;
         if (last >= 0) {
             const int32_t done = nt - (last + 1) * kKeyGroupTiles;  // steps the loop has taken for this group
-            for (int32_t step = done < 0 ? 0 : done; step < kDrainSteps; ++step) {
-                if (step % kLoaders == me) {
-                    drain_keys(kd, last, step, lane);
-                }
-            }
+            drain_tail(kd, last, done < 0 ? 0 : done, me, lane);
         }
     }
 }
@@ -497,9 +539,11 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     }
     // tiles [0, n_full) are those in which no request has run out of tokens
     const int32_t n_full = static_cast<int32_t>(full_u < ntiles_u ? full_u : ntiles_u);
+    // ... and of those, the ones whose keys may be staged (whole groups of them are)
+    const int32_t n_stageable = KS == kKeysSpread && ntiles_u < static_cast<uint32_t>(kSpreadFromTiles) ? 0 : n_full;
     if (wave != 0) {
         // ---------------------------------------------------------------- loader waves
-        const KeyDrain kd{s_keys, s_keypos, keys, n_full};
+        const KeyDrain kd{s_keys, s_keypos, keys, n_stageable};
         if (buffer_loads) {
             run_loader<BufferLoader<TokT>, TokT, KS>(ctx, s_tile, wave - 1, ntiles, lane, kd);
         } else {
@@ -534,7 +578,7 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         // a group of kKeyGroupTiles tiles is staged when all of its tiles are whole for every request; k and k + 1 lie
         // in the same group
         const int32_t group = k / kKeyGroupTiles;
-        const bool staged = KS && (group + 1) * kKeyGroupTiles <= n_full;
+        const bool staged = KS && (group + 1) * kKeyGroupTiles <= n_stageable;
         uint64_t *staged_row = KS ? s_keys + ((group & 1) * kReqs + lane) * kKeyRow + (k & (kKeyGroupTiles - 1)) * (kTT / 16)
                                   : nullptr;
         if (KS && staged) {
@@ -706,16 +750,19 @@ std::atomic<int32_t> g_force_global_loads{[] {
     return (fg && fg[0] == '1') ? 1 : 0;
 }()};
 
-// From how many requests in one launch the keys of 16-token blocks are staged in LDS and written by the loader waves
-// (hash_tokens_kernel<.., KS>), spread over the tiles or a group at a time. Chosen from timings on tokens that are not
-// in the memory-side cache, us for requests of 4096 tokens, direct / spread / burst:
-//   8-byte tokens   1024: 61 / 59 / 63    4096: 65 / 61 / 64     8192: 76 / 68 / 70      10 240: 83 / 76 / 73
-//                   12 288: 92 / 85 / 83  16 384: 112 / 111 / 107    32 768: 227 / 219 / 209
+// How the keys of 16-token blocks reach memory, by token width and number of requests in the launch
+// (hash_tokens_kernel<.., KS>). Chosen from timings on tokens that are not in the memory-side cache, us for requests of
+// 4096 tokens, direct / spread / burst:
+//   8-byte tokens   64: 61 / 58 / 60      1024: 61 / 59 / 63     4096: 65 / 60 / 64      8192: 76 / 64 / 70
+//                   10 240: 83 / 76 / 73  12 288: 92 / 85 / 83   16 384: 112 / 111 / 107   32 768: 227 / 219 / 209
 //   4-byte tokens   4096: 56 / 58 / 63    8192: 58 / 58 / 64     10 240: 64 / 62 / 66    12 288: 72 / 66 / 67
 //                   16 384: 85 / 81 / 78  32 768: 159 / 151 / 151
-// (4-byte tokens never take the spread form: two of the three are enough code.)
+// 8-byte tokens: direct below 2048 requests (there the spread form gains 2 to 4 % on tokens from HBM and loses as much
+// on resident ones, and costs requests of 1024 tokens 6 %), spread from 2048, burst from 10 240.
+// 4-byte tokens: direct below 12 288, burst from there (the spread form would gain 3 % between 10 240 and 16 384
+// requests: not worth one more kernel).
 #ifndef KVCM_HASH_SPREAD_FROM_8
-#define KVCM_HASH_SPREAD_FROM_8 4096
+#define KVCM_HASH_SPREAD_FROM_8 2048
 #endif
 #ifndef KVCM_HASH_BURST_FROM_8
 #define KVCM_HASH_BURST_FROM_8 10240

@@ -163,13 +163,15 @@ def test_bad_buffers_are_refused_on_the_host():
 
 @pytest.mark.parametrize("dtype", [np.int64, np.int32])
 @pytest.mark.parametrize("shape", ["uniform", "uniform_odd_count", "ragged", "ragged_short", "two_lengths",
-                                   "workgroup_on_every_cu", "every_cu_ragged", "every_cu_two_lengths"])
+                                   "workgroup_on_every_cu", "every_cu_ragged", "every_cu_two_lengths",
+                                   "short_and_long_workgroups"])
 def test_many_requests_take_the_staged_key_path(oracle, dtype, shape):
     """In launches of thousands of requests the keys of 16-token blocks are collected in LDS and written out as
-    512-byte rows by the loader waves: a sixteenth of a group per tile and the rest after the loop (8-byte tokens, 4096
-    to 10 239 requests), or a whole group right after the barrier that closes it (8-byte tokens from 10 240 requests,
-    4-byte tokens from 12 288). Groups of tiles in which some request has run out, requests past a multiple of 64, and
-    whatever does not fill a group of sixteen tiles go the direct way. Every mixture against the oracle, exact."""
+    512-byte rows by the loader waves: a sixteenth of a group per tile and the rest after the loop (8-byte tokens, 2048
+    to 10 239 requests; workgroups whose requests are shorter than 32 tiles store directly), or a whole group right
+    after the barrier that closes it (8-byte tokens from 10 240 requests, 4-byte tokens from 12 288). Groups of tiles in
+    which some request has run out, requests past a multiple of 64, and whatever does not fill a group of sixteen tiles
+    go the direct way. Every mixture against the oracle, exact."""
     rng = np.random.default_rng(5)
     lens = {
         "uniform": np.full(8192, 2048),                                # two whole groups per request
@@ -180,6 +182,8 @@ def test_many_requests_take_the_staged_key_path(oracle, dtype, shape):
         "workgroup_on_every_cu": np.full(16384 + 70, 1024 + 100),      # one group + a tile + a tail; last workgroup partial
         "every_cu_ragged": rng.integers(1100, 3000, size=16384 + 70),
         "every_cu_two_lengths": np.where(np.arange(16384) % 64 < 32, 3072, 1024),
+        # workgroups of short requests (direct), of long ones (staged) and of both in one launch of the spread kernel
+        "short_and_long_workgroups": np.where((np.arange(4096) // 64) % 3 == 0, 1536, np.where(np.arange(4096) % 5 == 0, 1024, 2560)),
     }[shape].astype(np.int64)
     toff = np.zeros(len(lens) + 1, dtype=np.int64)
     np.cumsum(lens, out=toff[1:])
