@@ -217,3 +217,31 @@ def test_staged_keys_with_the_general_loader(oracle, force_general_hash_loader, 
     sync()
     assert (host(keys, np.int64) == want).all()
 
+
+
+@pytest.mark.parametrize("dtype,R", [(np.int64, 2048 + 9), (np.int64, 10240 + 9), (np.int32, 12288 + 9), (np.int64, 2047)])
+def test_key_offsets_with_gaps_and_odd_starts(oracle, dtype, R):
+    """Keys go where key_offsets says, wherever that is: odd first positions (a request's 512-byte rows then start on
+    8-byte boundaries only) and gaps between the requests' ranges, which must stay untouched -- on both sides of the
+    request counts at which the way keys are written changes."""
+    rng = np.random.default_rng(31)
+    lens = rng.integers(2100, 2300, size=R).astype(np.int64)
+    lens[::7] = 1024 + 48                                                # some requests end early in every workgroup
+    toff = np.zeros(R + 1, dtype=np.int64)
+    np.cumsum(lens, out=toff[1:])
+    flat = rng.integers(-2**31, 2**31 - 1, size=int(toff[-1]), dtype=np.int64).astype(dtype)
+    want, woff = oracle.hash_tokens(flat, 16, token_offsets=toff, seed=-5, threads=8)
+    counts = lens // 16
+    gaps = rng.integers(0, 4, size=R)
+    koff = np.zeros(R + 1, dtype=np.int64)
+    koff[0] = 1
+    koff[1:] = 1 + np.cumsum(counts + gaps)
+    print(f"gapped key offsets: {R} requests of {np.dtype(dtype).name}, {int(koff[-1])} key slots", flush=True)
+    keys = torch.full((int(koff[-1]) + 64,), -7, dtype=torch.int64, device="cuda")
+    got, _ = _h().hash_tokens(dev(flat), 16, token_offsets=dev(toff), seed=-5, keys=keys, key_offsets=dev(koff))
+    sync()
+    got = host(got, np.int64)
+    expect = np.full(got.shape, -7, dtype=np.int64)
+    for r in range(R):
+        expect[koff[r]:koff[r] + counts[r]] = want[woff[r]:woff[r + 1]]
+    assert (got == expect).all()
