@@ -45,10 +45,13 @@ constexpr int kRing = 2;                      // LDS tiles in the ring: prefetch
                                               // computed on already sits in the chain wave's registers)
 constexpr int kPad = 2;                       // keeps rows 16-byte aligned (b128 reads) and spreads banks
 constexpr int kPerLane = kReqs * kTT / 64;  // tile elements per loader lane
-// Staged keys (many requests in flight, block size 16): the keys of kKeyGroupTiles tiles collect in LDS and leave as
-// whole rows of 512 bytes per request, see hash_tokens_kernel.
-constexpr int kKeyGroupTiles = 16;
-constexpr int kKeysPerGroup = kKeyGroupTiles * (kTT / 16);
+// Staged keys (many requests in flight; block sizes 1, 8, 16, 32 and 64): the keys of a GROUP of tiles collect in LDS
+// and leave as whole rows of 512 bytes per request, see hash_tokens_kernel. A group is as many tiles as yield 64 keys per
+// request: key_group_tiles(block size), i.e. one tile at block size 1 and sixteen at block size 16.
+constexpr int kKeysPerGroup = 64;
+constexpr int key_group_tiles(int bs) { return bs >= 1 && bs <= kTT ? kKeysPerGroup / (kTT / bs) : 16; }
+constexpr int kKeyGroupTiles = key_group_tiles(16);  // the spread form exists for block size 16 only
+static_assert(key_group_tiles(1) == 1 && key_group_tiles(16) == 16 && key_group_tiles(64) == 64, "64 keys per group");
 constexpr int kKeyPad = 2;
 constexpr int kKeyRow = kKeysPerGroup + kKeyPad;  // one request's row of the LDS key buffer
 
@@ -336,10 +339,11 @@ __device__ __forceinline__ void drain_tail(const KeyDrain &kd, int32_t group, in
     }
 }
 
-template <typename Loader, typename TokT, int KS>
+template <typename Loader, typename TokT, int KS, int G>
 __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t (*s_tile)[kReqs][kTT + kPad],
                                            int64_t lw, int64_t ntiles, uint32_t lane, const KeyDrain &kd) {
     static_assert(kRing == 2 && kLoaders >= 3, "two ring slots: prefetched from, written to");
+    static_assert((G & (G - 1)) == 0 && (KS != kKeysSpread || G == kKeyGroupTiles), "groups of 2^n tiles; spread: 16");
     Loader ld;
     ld.setup(ctx, lane);
     // 32-bit counters: the loop control stays in scalar registers (there are no ordered 64-bit scalar compares); a
@@ -396,10 +400,10 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
             }
         }
         was_mine = mine;
-        if (KS == kKeysBurst && (k & (kKeyGroupTiles - 1)) == kKeyGroupTiles - 1 && k < kd.full_tiles && turn != me) {
-            // The barrier above closed a group. The loader whose tile is due next leaves it alone (its next wait for
-            // memory would wait for these stores as well); the other two write half of it each.
-            drain_half(kd, k / kKeyGroupTiles, (me - turn + kLoaders) % kLoaders - 1, lane);
+        if (KS == kKeysBurst && (k & (G - 1)) == G - 1 && k < kd.full_tiles && turn != me) {
+            // The barrier above closed a group of G tiles. The loader whose tile is due next leaves it alone (its next
+            // wait for memory would wait for these stores as well); the other two write half of it each.
+            drain_half(kd, k / G, (me - turn + kLoaders) % kLoaders - 1, lane);
         }
     }
     if (KS == kKeysSpread) {
@@ -421,13 +425,13 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
 // BS > 0 = the block size is this compile-time constant (a divisor or a multiple of the tile): the places where a key
 // is due are then known when the code is written, and the scalar bookkeeping (add, compare, branch per chunk: one
 // instruction slot in sixteen of the wave that sets the pace) disappears from the loop.
-// STAGED (unmasked tiles, block size 16): the tile's keys go to the lane's row of the LDS key buffer, `staged_row`
+// STAGED (unmasked tiles, block size a compile-time constant up to a tile): the tile's keys go to the lane's row of the LDS key buffer, `staged_row`
 // pointing at the tile's first key there; a loader wave writes the rows out (drain_keys).
 template <int CHUNK, bool MASKED, int BS, bool STAGED = false>
 __device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_t &h, int64_t t0, int64_t my_ntok,
                                          int32_t &since_key, int32_t block_size, int64_t *__restrict__ keys,
                                          int64_t &key_pos, uint64_t *staged_row = nullptr) {
-    static_assert(!STAGED || (!MASKED && BS == 16), "keys are staged for whole tiles of 16-token blocks only");
+    static_assert(!STAGED || (!MASKED && BS >= 1 && BS <= kTT), "keys are staged for whole tiles of blocks up to a tile");
     static_assert(BS == 0 || (BS % CHUNK == 0 && (kTT % BS == 0 || BS % kTT == 0)), "block size fits the tiling");
     // tokens of this lane that are hashed and lie in this tile or before its end: a block that ends at position p of
     // the tile belongs to the lane iff p <= left (my_ntok is a multiple of the block size)
@@ -472,10 +476,10 @@ __device__ __forceinline__ void read_row(ulonglong2 (&a)[kTT / 2], const uint64_
 
 // CHUNK = steps between two looks at the block boundary: 8 when block_size % 8 == 0 (a lane is then
 // active for whole chunks or not at all), otherwise 1. BS = block size when it is 1, 8, 16, 32, 64 or 128, otherwise 0.
-// KS != kKeysDirect ("keys staged", block size 16 only; chosen by the host for batches of many requests, where the launch
+// KS != kKeysDirect ("keys staged", block sizes 1 to 64; chosen by the host for batches of many requests, where the launch
 // is bound by memory and not by the chain): the chain wave writes its keys into an LDS buffer instead of to memory, and
-// after every kKeyGroupTiles tiles in which every request is whole the loader waves write the group out as rows of 512
-// bytes, spread over the next group's tiles or at once.
+// after every group of tiles in which every request is whole the loader waves write the group out as rows of 512
+// bytes, spread over the next group's tiles (block size 16) or at once.
 template <typename TokT, int CHUNK, int BS, int KS = kKeysDirect>
 __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__restrict__ tokens,
                                                               const int64_t *__restrict__ token_offsets, int32_t R,
@@ -486,7 +490,10 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     __shared__ __attribute__((aligned(16))) uint64_t s_tile[kRing][kReqs][kTT + kPad];
     __shared__ int64_t s_start[kReqs];
     __shared__ int64_t s_ntok[kReqs];
-    static_assert(!KS || BS == 16, "keys are staged for 16-token blocks");
+    static_assert(!KS || (BS >= 1 && BS <= kTT), "keys are staged for block sizes up to a tile");
+    static_assert(KS != kKeysSpread || BS == 16, "the spread form exists for 16-token blocks");
+    constexpr int G = key_group_tiles(BS);  // tiles per group of staged keys
+    constexpr int kKeysPerTile = KS ? kTT / (BS > 0 ? BS : 1) : 0;
     __shared__ __attribute__((aligned(16))) uint64_t s_keys[KS ? 2 * kReqs * kKeyRow : 2];
     __shared__ int64_t s_keypos[KS ? kReqs : 1];
 
@@ -545,9 +552,9 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         // ---------------------------------------------------------------- loader waves
         const KeyDrain kd{s_keys, s_keypos, keys, n_stageable};
         if (buffer_loads) {
-            run_loader<BufferLoader<TokT>, TokT, KS>(ctx, s_tile, wave - 1, ntiles, lane, kd);
+            run_loader<BufferLoader<TokT>, TokT, KS, G>(ctx, s_tile, wave - 1, ntiles, lane, kd);
         } else {
-            run_loader<GlobalLoader<TokT>, TokT, KS>(ctx, s_tile, wave - 1, ntiles, lane, kd);
+            run_loader<GlobalLoader<TokT>, TokT, KS, G>(ctx, s_tile, wave - 1, ntiles, lane, kd);
         }
         return;
     }
@@ -575,12 +582,10 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         if (k + 1 < nt) {
             read_row(nxt, &s_tile[ring1][lane][0]);
         }
-        // a group of kKeyGroupTiles tiles is staged when all of its tiles are whole for every request; k and k + 1 lie
-        // in the same group
-        const int32_t group = k / kKeyGroupTiles;
-        const bool staged = KS && (group + 1) * kKeyGroupTiles <= n_stageable;
-        uint64_t *staged_row = KS ? s_keys + ((group & 1) * kReqs + lane) * kKeyRow + (k & (kKeyGroupTiles - 1)) * (kTT / 16)
-                                  : nullptr;
+        // a group of G tiles is staged when all of its tiles are whole for every request
+        const int32_t group = k / G;
+        const bool staged = KS && (group + 1) * G <= n_stageable;
+        uint64_t *staged_row = KS ? s_keys + ((group & 1) * kReqs + lane) * kKeyRow + (k & (G - 1)) * kKeysPerTile : nullptr;
         if (KS && staged) {
             run_tile<CHUNK, false, BS, KS != kKeysDirect>(cur, h, static_cast<int64_t>(k) * kTT, my_ntok, since_key, block_size, keys,
                                            key_pos, staged_row);
@@ -599,9 +604,13 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         if (k + 2 < nt) {
             read_row(cur, &s_tile[ring][lane][0]);
         }
-        if (KS && staged) {
+        const int32_t group1 = (k + 1) / G;  // the same group unless a group is one tile
+        const bool staged1 = KS && (group1 + 1) * G <= n_stageable;
+        uint64_t *staged_row1 =
+            KS ? s_keys + ((group1 & 1) * kReqs + lane) * kKeyRow + ((k + 1) & (G - 1)) * kKeysPerTile : nullptr;
+        if (KS && staged1) {
             run_tile<CHUNK, false, BS, KS != kKeysDirect>(nxt, h, static_cast<int64_t>(k + 1) * kTT, my_ntok, since_key, block_size,
-                                           keys, key_pos, staged_row + kTT / 16);
+                                           keys, key_pos, staged_row1);
         } else if (k + 1 < n_full) {
             run_tile<CHUNK, false, BS>(nxt, h, static_cast<int64_t>(k + 1) * kTT, my_ntok, since_key, block_size, keys,
                                        key_pos);
@@ -750,9 +759,9 @@ std::atomic<int32_t> g_force_global_loads{[] {
     return (fg && fg[0] == '1') ? 1 : 0;
 }()};
 
-// How the keys of 16-token blocks reach memory, by token width and number of requests in the launch
-// (hash_tokens_kernel<.., KS>). Chosen from timings on tokens that are not in the memory-side cache, us for requests of
-// 4096 tokens, direct / spread / burst:
+// How keys reach memory, by block size, token width and number of requests in the launch (hash_tokens_kernel<.., KS>).
+// Chosen from timings on tokens that are not in the memory-side cache. 16-token blocks, us for requests of 4096 tokens,
+// direct / spread / burst:
 //   8-byte tokens   64: 61 / 58 / 60      1024: 61 / 59 / 63     4096: 65 / 60 / 64      8192: 76 / 64 / 70
 //                   10 240: 83 / 76 / 73  12 288: 92 / 85 / 83   16 384: 112 / 111 / 107   32 768: 227 / 219 / 209
 //   4-byte tokens   4096: 56 / 58 / 63    8192: 58 / 58 / 64     10 240: 64 / 62 / 66    12 288: 72 / 66 / 67
@@ -761,14 +770,31 @@ std::atomic<int32_t> g_force_global_loads{[] {
 // on resident ones, and costs requests of 1024 tokens 6 %), spread from 2048, burst from 10 240.
 // 4-byte tokens: direct below 12 288, burst from there (the spread form would gain 3 % between 10 240 and 16 384
 // requests: not worth one more kernel).
+// Other block sizes, direct / burst:
+//   block size 1, 8-byte tokens   64: 146 / 129   2048: 158 / 136   8192: 241 / 161   16 384: 300 / 202   32 768: 641 / 415
+//                 4-byte tokens   512: 115 / 119  1024: 119 / 120 (resident: 116 / 92)   8192: 184 / 141   16 384: 249 / 175
+//   block size 8, 8-byte tokens   1024: 72 / 69 (resident: 61 / 64)   2048: 74 / 70   8192: 98 / 77   16 384: 137 / 112
+//                 4-byte tokens   8192: 69 / 71   12 288: 82 / 75   16 384: 100 / 83
+//   block size 32, 8-byte tokens  4096: 60 / 61   8192: 69 / 65   12 288: 93 / 76   16 384: 115 / 99
+//                  4-byte tokens  8192: 57 / 57   12 288: 69 / 62   16 384: 84 / 70
+//   block size 64, 8-byte tokens  4096: 58 / 60   8192: 67 / 63   12 288: 85 / 75   16 384: 109 / 93
+//                  4-byte tokens  8192: 55 / 57   12 288: 64 / 60   16 384: 77 / 72
 #ifndef KVCM_HASH_SPREAD_FROM_8
 #define KVCM_HASH_SPREAD_FROM_8 2048
 #endif
-#ifndef KVCM_HASH_BURST_FROM_8
-#define KVCM_HASH_BURST_FROM_8 10240
-#endif
-#ifndef KVCM_HASH_BURST_FROM_4
-#define KVCM_HASH_BURST_FROM_4 12288
+// requests from which a launch takes the burst form; INT32_MAX = never
+constexpr int32_t burst_from(int32_t block_size, bool tokens_8_byte) {
+    switch (block_size) {
+        case 1: return tokens_8_byte ? 1 : 1024;
+        case 8: return tokens_8_byte ? 2048 : 12288;
+        case 16: return tokens_8_byte ? 10240 : 12288;
+        case 32: return tokens_8_byte ? 8192 : 12288;
+        case 64: return tokens_8_byte ? 8192 : 12288;
+        default: return INT32_MAX;
+    }
+}
+#ifndef KVCM_HASH_BURST_SCALE  // for experiments: 0 = burst wherever it exists, a large number = never
+#define KVCM_HASH_BURST_SCALE 1
 #endif
 
 template <typename TokT>
@@ -789,29 +815,47 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
     hipLaunchKernelGGL((hash_tokens_kernel<TokT, CHUNK, BS>), grid, dim3(kThreads), 0, stream, d_tokens,            \
                        d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
     constexpr bool k8 = sizeof(TokT) == 8;
-    const bool burst = block_size == 16 && R >= (k8 ? KVCM_HASH_BURST_FROM_8 : KVCM_HASH_BURST_FROM_4);
+    const bool burst = R >= static_cast<int64_t>(burst_from(block_size, k8)) * KVCM_HASH_BURST_SCALE;
     const bool spread = block_size == 16 && k8 && !burst && R >= KVCM_HASH_SPREAD_FROM_8;
-#define KVCM_LAUNCH_HASH_STAGED(KS)                                                                                  \
-    hipLaunchKernelGGL((hash_tokens_kernel<TokT, 8, 16, KS>), grid, dim3(kThreads), 0, stream, d_tokens,            \
+#define KVCM_LAUNCH_HASH_STAGED(CHUNK, BS, KS)                                                                       \
+    hipLaunchKernelGGL((hash_tokens_kernel<TokT, CHUNK, BS, KS>), grid, dim3(kThreads), 0, stream, d_tokens,        \
                        d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
-    if (burst) {
-        KVCM_LAUNCH_HASH_STAGED(kKeysBurst);
-    } else if (spread) {
+    if (spread) {
         if constexpr (k8) {
-            KVCM_LAUNCH_HASH_STAGED(kKeysSpread);
+            KVCM_LAUNCH_HASH_STAGED(8, 16, kKeysSpread);
         }
     } else if (block_size == 16) {  // the engines' usual block sizes get kernels of their own
-        KVCM_LAUNCH_HASH(8, 16);
+        if (burst) {
+            KVCM_LAUNCH_HASH_STAGED(8, 16, kKeysBurst);
+        } else {
+            KVCM_LAUNCH_HASH(8, 16);
+        }
     } else if (block_size == 8) {
-        KVCM_LAUNCH_HASH(8, 8);
+        if (burst) {
+            KVCM_LAUNCH_HASH_STAGED(8, 8, kKeysBurst);
+        } else {
+            KVCM_LAUNCH_HASH(8, 8);
+        }
     } else if (block_size == 32) {
-        KVCM_LAUNCH_HASH(8, 32);
+        if (burst) {
+            KVCM_LAUNCH_HASH_STAGED(8, 32, kKeysBurst);
+        } else {
+            KVCM_LAUNCH_HASH(8, 32);
+        }
     } else if (block_size == 64) {
-        KVCM_LAUNCH_HASH(8, 64);
+        if (burst) {
+            KVCM_LAUNCH_HASH_STAGED(8, 64, kKeysBurst);
+        } else {
+            KVCM_LAUNCH_HASH(8, 64);
+        }
     } else if (block_size == 128) {
         KVCM_LAUNCH_HASH(8, 128);
     } else if (block_size == 1) {  // the prefix chain over digests: a key after every step
-        KVCM_LAUNCH_HASH(1, 1);
+        if (burst) {
+            KVCM_LAUNCH_HASH_STAGED(1, 1, kKeysBurst);
+        } else {
+            KVCM_LAUNCH_HASH(1, 1);
+        }
     } else if (block_size % 8 == 0) {
         KVCM_LAUNCH_HASH(8, 0);
     } else {

@@ -201,8 +201,9 @@ def test_many_requests_take_the_staged_key_path(oracle, dtype, shape):
     assert (host(got, np.int64)[len(want):] == -7).all()
 
 
-@pytest.mark.parametrize("dtype,R", [(np.int64, 16384 + 70), (np.int64, 8300), (np.int32, 12288 + 70)])
-def test_staged_keys_with_the_general_loader(oracle, force_general_hash_loader, dtype, R):
+@pytest.mark.parametrize("dtype,R,bs", [(np.int64, 16384 + 70, 16), (np.int64, 8300, 16), (np.int32, 12288 + 70, 16),
+                                         (np.int64, 300, 1), (np.int64, 2100, 8)])
+def test_staged_keys_with_the_general_loader(oracle, force_general_hash_loader, dtype, R, bs):
     """The staged-key forms (spread and burst) are loader code as well: both with the loader that a workgroup spanning
     4 GiB of tokens would take, ragged requests, exact."""
     force_general_hash_loader(True)
@@ -211,9 +212,9 @@ def test_staged_keys_with_the_general_loader(oracle, force_general_hash_loader, 
     toff = np.zeros(R + 1, dtype=np.int64)
     np.cumsum(lens, out=toff[1:])
     flat = rng.integers(-2**31, 2**31 - 1, size=int(toff[-1]), dtype=np.int64).astype(dtype)
-    print(f"staged keys, general loader: {R} requests of {np.dtype(dtype).name}, {int(toff[-1])} tokens", flush=True)
-    want, woff = oracle.hash_tokens(flat, 16, token_offsets=toff, threads=8)
-    keys, off = _h().hash_tokens(dev(flat), 16, token_offsets=dev(toff))
+    print(f"staged keys, general loader: {R} requests of {np.dtype(dtype).name}, block size {bs}, {int(toff[-1])} tokens", flush=True)
+    want, woff = oracle.hash_tokens(flat, bs, token_offsets=toff, threads=8)
+    keys, off = _h().hash_tokens(dev(flat), bs, token_offsets=dev(toff))
     sync()
     assert (host(keys, np.int64) == want).all()
 
@@ -245,3 +246,27 @@ def test_key_offsets_with_gaps_and_odd_starts(oracle, dtype, R):
     for r in range(R):
         expect[koff[r]:koff[r] + counts[r]] = want[woff[r]:woff[r + 1]]
     assert (got == expect).all()
+
+
+@pytest.mark.parametrize("bs,dtype", [(1, np.int64), (8, np.int64), (32, np.int64), (64, np.int64), (8, np.int32),
+                                      (1, np.int32)])
+def test_staged_keys_at_other_block_sizes(oracle, bs, dtype):
+    """In launches of many requests the keys of 1-, 8-, 32- and 64-token blocks are staged too (a group is as many
+    tiles as yield 64 keys per request: 1, 8, 32, 64 tiles) and leave a group at a time. Ragged requests of one to three
+    groups, some ending early, the last workgroup partial; exact against the oracle, spare key slots untouched."""
+    group_tokens = 64 * max(bs, 1) if bs > 1 else 64
+    rng = np.random.default_rng(41 + bs)
+    R = (10240 if dtype == np.int64 else 12288) + 37   # past every threshold of the launch rule
+    lens = rng.integers(group_tokens + 70, 3 * group_tokens, size=R).astype(np.int64)
+    lens[::9] = group_tokens // 2 + 5
+    toff = np.zeros(R + 1, dtype=np.int64)
+    np.cumsum(lens, out=toff[1:])
+    flat = rng.integers(-2**31, 2**31 - 1, size=int(toff[-1]), dtype=np.int64).astype(dtype)
+    print(f"staged keys, block size {bs}: {R} requests of {np.dtype(dtype).name}, {int(toff[-1])} tokens", flush=True)
+    want, woff = oracle.hash_tokens(flat, bs, token_offsets=toff, seed=11, threads=8)
+    keys = torch.full((len(want) + 64,), -7, dtype=torch.int64, device="cuda")
+    got, off = _h().hash_tokens(dev(flat), bs, token_offsets=dev(toff), seed=11, keys=keys, key_offsets=dev(woff))
+    sync()
+    got = host(got, np.int64)
+    assert (got[:len(want)] == want).all()
+    assert (got[len(want):] == -7).all()
