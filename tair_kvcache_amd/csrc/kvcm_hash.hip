@@ -45,13 +45,13 @@ constexpr int kRing = 2;                      // LDS tiles in the ring: prefetch
                                               // computed on already sits in the chain wave's registers)
 constexpr int kPad = 2;                       // keeps rows 16-byte aligned (b128 reads) and spreads banks
 constexpr int kPerLane = kReqs * kTT / 64;  // tile elements per loader lane
-// Staged keys (many requests in flight; block sizes 1, 8, 16, 32 and 64): the keys of a GROUP of tiles collect in LDS
+// Staged keys (many requests in flight; block sizes 1, 8, 16, 32, 64 and 128): the keys of a GROUP of tiles collect in LDS
 // and leave as whole rows of 512 bytes per request, see hash_tokens_kernel. A group is as many tiles as yield 64 keys per
-// request: key_group_tiles(block size), i.e. one tile at block size 1 and sixteen at block size 16.
+// request: key_group_tiles(block size), i.e. one tile at block size 1, sixteen at block size 16, 128 at block size 128.
 constexpr int kKeysPerGroup = 64;
-constexpr int key_group_tiles(int bs) { return bs >= 1 && bs <= kTT ? kKeysPerGroup / (kTT / bs) : 16; }
+constexpr int key_group_tiles(int bs) { return bs >= 1 && bs <= 2 * kTT ? kKeysPerGroup * bs / kTT : 16; }
 constexpr int kKeyGroupTiles = key_group_tiles(16);  // the spread form exists for block size 16 only
-static_assert(key_group_tiles(1) == 1 && key_group_tiles(16) == 16 && key_group_tiles(64) == 64, "64 keys per group");
+static_assert(key_group_tiles(1) == 1 && key_group_tiles(16) == 16 && key_group_tiles(128) == 128, "64 keys per group");
 constexpr int kKeyPad = 2;
 constexpr int kKeyRow = kKeysPerGroup + kKeyPad;  // one request's row of the LDS key buffer
 
@@ -431,7 +431,7 @@ template <int CHUNK, bool MASKED, int BS, bool STAGED = false>
 __device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_t &h, int64_t t0, int64_t my_ntok,
                                          int32_t &since_key, int32_t block_size, int64_t *__restrict__ keys,
                                          int64_t &key_pos, uint64_t *staged_row = nullptr) {
-    static_assert(!STAGED || (!MASKED && BS >= 1 && BS <= kTT), "keys are staged for whole tiles of blocks up to a tile");
+    static_assert(!STAGED || (!MASKED && BS >= 1 && BS <= 2 * kTT), "keys are staged for whole tiles of blocks up to two tiles");
     static_assert(BS == 0 || (BS % CHUNK == 0 && (kTT % BS == 0 || BS % kTT == 0)), "block size fits the tiling");
     // tokens of this lane that are hashed and lie in this tile or before its end: a block that ends at position p of
     // the tile belongs to the lane iff p <= left (my_ntok is a multiple of the block size)
@@ -457,7 +457,7 @@ __device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_
         }
         if (key_due) {
             if (STAGED) {
-                staged_row[(c + CHUNK) / (BS > 0 ? BS : 1) - 1] = h;
+                staged_row[BS > kTT ? 0 : (c + CHUNK) / (BS > 0 ? BS : 1) - 1] = h;
             } else if (!MASKED || c + CHUNK <= left) {
                 keys[key_pos] = static_cast<int64_t>(h);
             }
@@ -490,10 +490,10 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     __shared__ __attribute__((aligned(16))) uint64_t s_tile[kRing][kReqs][kTT + kPad];
     __shared__ int64_t s_start[kReqs];
     __shared__ int64_t s_ntok[kReqs];
-    static_assert(!KS || (BS >= 1 && BS <= kTT), "keys are staged for block sizes up to a tile");
+    static_assert(!KS || (BS >= 1 && BS <= 2 * kTT), "keys are staged for block sizes up to two tiles");
     static_assert(KS != kKeysSpread || BS == 16, "the spread form exists for 16-token blocks");
     constexpr int G = key_group_tiles(BS);  // tiles per group of staged keys
-    constexpr int kKeysPerTile = KS ? kTT / (BS > 0 ? BS : 1) : 0;
+    constexpr int kDiv = BS > 0 ? BS : 1;  // the first key of tile t of a group lies at position t * kTT / BS of the row
     __shared__ __attribute__((aligned(16))) uint64_t s_keys[KS ? 2 * kReqs * kKeyRow : 2];
     __shared__ int64_t s_keypos[KS ? kReqs : 1];
 
@@ -585,7 +585,7 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         // a group of G tiles is staged when all of its tiles are whole for every request
         const int32_t group = k / G;
         const bool staged = KS && (group + 1) * G <= n_stageable;
-        uint64_t *staged_row = KS ? s_keys + ((group & 1) * kReqs + lane) * kKeyRow + (k & (G - 1)) * kKeysPerTile : nullptr;
+        uint64_t *staged_row = KS ? s_keys + ((group & 1) * kReqs + lane) * kKeyRow + (k & (G - 1)) * kTT / kDiv : nullptr;
         if (KS && staged) {
             run_tile<CHUNK, false, BS, KS != kKeysDirect>(cur, h, static_cast<int64_t>(k) * kTT, my_ntok, since_key, block_size, keys,
                                            key_pos, staged_row);
@@ -607,7 +607,7 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         const int32_t group1 = (k + 1) / G;  // the same group unless a group is one tile
         const bool staged1 = KS && (group1 + 1) * G <= n_stageable;
         uint64_t *staged_row1 =
-            KS ? s_keys + ((group1 & 1) * kReqs + lane) * kKeyRow + ((k + 1) & (G - 1)) * kKeysPerTile : nullptr;
+            KS ? s_keys + ((group1 & 1) * kReqs + lane) * kKeyRow + ((k + 1) & (G - 1)) * kTT / kDiv : nullptr;
         if (KS && staged1) {
             run_tile<CHUNK, false, BS, KS != kKeysDirect>(nxt, h, static_cast<int64_t>(k + 1) * kTT, my_ntok, since_key, block_size,
                                            keys, key_pos, staged_row1);
@@ -779,6 +779,8 @@ std::atomic<int32_t> g_force_global_loads{[] {
 //                  4-byte tokens  8192: 57 / 57   12 288: 69 / 62   16 384: 84 / 70
 //   block size 64, 8-byte tokens  4096: 58 / 60   8192: 67 / 63   12 288: 85 / 75   16 384: 109 / 93
 //                  4-byte tokens  8192: 55 / 57   12 288: 64 / 60   16 384: 77 / 72
+//   block size 128 (requests of 16 384 tokens: a group is 8192), 8-byte tokens  4096: 210 / 208   8192: 242 / 222
+//                  16 384: 419 / 356;  4-byte tokens  8192: 198 / 197   16 384: 264 / 204
 #ifndef KVCM_HASH_SPREAD_FROM_8
 #define KVCM_HASH_SPREAD_FROM_8 2048
 #endif
@@ -790,6 +792,7 @@ constexpr int32_t burst_from(int32_t block_size, bool tokens_8_byte) {
         case 16: return tokens_8_byte ? 10240 : 12288;
         case 32: return tokens_8_byte ? 8192 : 12288;
         case 64: return tokens_8_byte ? 8192 : 12288;
+        case 128: return tokens_8_byte ? 8192 : 12288;
         default: return INT32_MAX;
     }
 }
@@ -849,7 +852,11 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
             KVCM_LAUNCH_HASH(8, 64);
         }
     } else if (block_size == 128) {
-        KVCM_LAUNCH_HASH(8, 128);
+        if (burst) {
+            KVCM_LAUNCH_HASH_STAGED(8, 128, kKeysBurst);
+        } else {
+            KVCM_LAUNCH_HASH(8, 128);
+        }
     } else if (block_size == 1) {  // the prefix chain over digests: a key after every step
         if (burst) {
             KVCM_LAUNCH_HASH_STAGED(1, 1, kKeysBurst);

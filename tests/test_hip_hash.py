@@ -249,15 +249,15 @@ def test_key_offsets_with_gaps_and_odd_starts(oracle, dtype, R):
 
 
 @pytest.mark.parametrize("bs,dtype", [(1, np.int64), (8, np.int64), (32, np.int64), (64, np.int64), (8, np.int32),
-                                      (1, np.int32)])
+                                      (1, np.int32), (128, np.int64)])
 def test_staged_keys_at_other_block_sizes(oracle, bs, dtype):
-    """In launches of many requests the keys of 1-, 8-, 32- and 64-token blocks are staged too (a group is as many
-    tiles as yield 64 keys per request: 1, 8, 32, 64 tiles) and leave a group at a time. Ragged requests of one to three
+    """In launches of many requests the keys of 1-, 8-, 32-, 64- and 128-token blocks are staged too (a group is as many
+    tiles as yield 64 keys per request: 1, 8, 32, 64, 128 tiles) and leave a group at a time. Ragged requests of one to three
     groups, some ending early, the last workgroup partial; exact against the oracle, spare key slots untouched."""
     group_tokens = 64 * max(bs, 1) if bs > 1 else 64
     rng = np.random.default_rng(41 + bs)
     R = (10240 if dtype == np.int64 else 12288) + 37   # past every threshold of the launch rule
-    lens = rng.integers(group_tokens + 70, 3 * group_tokens, size=R).astype(np.int64)
+    lens = rng.integers(group_tokens + 70, (3 if bs < 128 else 1.5) * group_tokens, size=R).astype(np.int64)
     lens[::9] = group_tokens // 2 + 5
     toff = np.zeros(R + 1, dtype=np.int64)
     np.cumsum(lens, out=toff[1:])
