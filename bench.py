@@ -38,8 +38,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # were measured on: a run whose sources differ reports traffic null and says why.
 KERNEL_SOURCES = ("tair_kvcache_amd/csrc/kvcm_copy.hip", "tair_kvcache_amd/csrc/kvcm_hash.hip",
                   "tair_kvcache_amd/csrc/kvcm_internal.h")
-MEASURED_TRAFFIC = {"sources_sha256": "ee3b93a191732161", "unique_blocks": 12416, "gather": 52076665853,
-                    "scatter": 52076191085, "hash_saturated": 571038104}
+MEASURED_TRAFFIC = {"sources_sha256": "72a535e858f36b02", "unique_blocks": 12416, "gather": 52076667576,
+                    "scatter": 52076193025, "hash_saturated": 571031008}
 
 # Llama-3-8B KV layout: the configuration the headline metric is quoted on
 LAYERS, KV_HEADS, HEAD_DIM, ITEMSIZE = 32, 8, 128, 2
@@ -171,7 +171,7 @@ def cold_ms(torch, fn, device, reps=7, sweep_gib=2):
 
 
 def other_configs(torch, np, device, reps=5):
-    """BASELINE configurations 1, 3, 4 and 5 at their full sizes, one after the other (memory is released in between):
+    """Benchmark configurations 1, 3, 4 and 5 (BASELINE.json) at their full sizes, one after the other (memory is released in between):
     save (gather) and load (scatter) milliseconds, GB/s of read+written bytes and the fraction of the HBM peak, and the
     block-key kernel at the configuration's own request count. A sample of every result is checked on the device."""
     from tair_kvcache_amd import _lib, hashing, save_selection

@@ -301,7 +301,7 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
             for (int u = 0; u < kCPT; ++u) {
                 if constexpr (CS == 16) {
                     // Block-table form (whole tiles move): the staging side of a gather is written through at system
-                    // scope (sc1), measured +1.5 to +4.6 % over non-temporal stores at the BASELINE layouts and +1.6 %
+                    // scope (sc1), measured +1.5 to +4.6 % over non-temporal stores at the benchmark layouts and +1.6 %
                     // for 128-block tasks; the pool side of a scatter carries sc1 and nt together (+1.3 to +2.5 %, and a
                     // 24 MiB launch that fits the caches finishes 45 % sooner). With token-granular indices either bit
                     // costs 0.5 to 2.5 %: those stores stay non-temporal. Where staging tiles do not start on cache-line

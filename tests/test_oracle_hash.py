@@ -56,7 +56,7 @@ def test_golden_prefix_chains_and_folds(oracle, golden):
         assert got.tolist() == [f["hash"]]
 
 
-def test_survey_known_answers(oracle):
+def test_known_answers_of_the_compiled_reference_header(oracle):
     keys = oracle.gen_key_vector(np.arange(64, dtype=np.int64), 16)
     assert [int(k) & M for k in keys] == [0x5AFC88D355FF4B7B, 0x10B81CF351F85B40, 0x9663CF74B462B173,
                                           0x253717686B900F1B]
