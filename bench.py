@@ -475,6 +475,12 @@ def main():
     ms_scatter = sum(e[2].elapsed_time(e[3]) for e in events) / args.steps
     ms_step = wall * 1e3 / args.steps
 
+    def spread(i):  # minimum and median over the steps, beside the average that the figures above are built on
+        v = sorted(e[i].elapsed_time(e[i + 1]) for e in events)
+        return {"min": round(v[0], 4), "median": round(v[len(v) // 2], 4), "max": round(v[-1], 4)}
+
+    per_step = {"hash_ms": spread(0), "save_ms": spread(1), "load_ms": spread(2)}
+
     if args.calibrate_copy_gib > 0:
         n = int(args.calibrate_copy_gib * 2**30)
         src = staging.view(torch.uint8).reshape(-1)[:n]
@@ -642,6 +648,7 @@ def main():
                    "requests": REQUESTS, "tokens_per_request": TOKENS_PER_REQ, "block_tokens": T},
         "save_GBps": roof_g["achieved"], "save_frac_of_hbm_peak": roof_g["frac"], "save_ms": round(ms_gather, 4),
         "load_GBps": roof_s["achieved"], "load_frac_of_hbm_peak": roof_s["frac"], "load_ms": round(ms_scatter, 4),
+        "per_step": per_step,
         "contiguous_copy_same_kernel": contiguous,
         "keys_per_s": round(d_keys.numel() / (ms_hash * 1e-3)), "hash_ms": round(ms_hash, 4), "hash_chains": REQUESTS,
         "hash_ms_back_to_back": round(ms_hash_b2b, 4),
