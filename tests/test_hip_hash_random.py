@@ -50,3 +50,37 @@ def test_random_batches(oracle, force_general_hash_loader, force_global):
             sync()
             assert (host(off, np.int64) == woff).all(), (i, rep)
             assert (host(keys, np.int64) == want).all(), (i, rep, R, bs, seed)
+
+
+def test_random_launches_of_many_requests(oracle):
+    """The same against the oracle for launches of thousands of requests, on both sides of every request count at which
+    the way keys reach memory changes, for the block sizes that have staged forms; lengths of one to a few groups of
+    tiles, ragged, some requests empty or short, key ranges with gaps."""
+    from tair_kvcache_amd import hashing
+    rng = np.random.default_rng(123)
+    for i in range(18):
+        bs = int(rng.choice([1, 8, 16, 16, 32, 64, 128]))
+        R = int(rng.choice([1023, 1024, 2047, 2048, 4100, 8191, 8192, 10239, 10240, 12287, 12288, 16390]))
+        dtype = np.int32 if rng.random() < 0.4 else np.int64
+        group_tokens = 64 * bs if bs > 1 else 64
+        top = int(min(max(2.5 * group_tokens, 300), 24_000_000 // R))
+        lens = rng.integers(top // 3, top + 1, size=R).astype(np.int64)
+        lens[rng.random(R) < 0.05] = rng.integers(0, 40)
+        toff = np.zeros(R + 1, dtype=np.int64)
+        np.cumsum(lens, out=toff[1:])
+        flat = rng.integers(-2**31, 2**31 - 1, size=int(toff[-1]), dtype=np.int64).astype(dtype)
+        seed = int(rng.choice([0, -1, 2**62]))
+        print(f"hash random large case {i}: R={R} lens {top // 3}..{top} bs={bs} seed={seed} {np.dtype(dtype).name}", flush=True)
+        want, woff = oracle.hash_tokens(flat, bs, token_offsets=toff, seed=seed, threads=8)
+        counts = lens // bs
+        koff = np.zeros(R + 1, dtype=np.int64)
+        koff[1:] = np.cumsum(counts + rng.integers(0, 3, size=R))
+        import torch
+        keys = torch.full((int(koff[-1]) + 16,), -7, dtype=torch.int64, device="cuda")
+        got, _ = hashing.hash_tokens(dev(flat), bs, token_offsets=dev(toff), seed=seed, keys=keys, key_offsets=dev(koff))
+        sync()
+        got = host(got, np.int64)
+        expect = np.full(got.shape, -7, dtype=np.int64)
+        idx = np.repeat(koff[:-1] - woff[:-1], counts) + np.arange(len(want))
+        expect[idx] = want
+        assert (got == expect).all(), (i, R, bs, seed)
