@@ -38,8 +38,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # were measured on: a run whose sources differ reports traffic null and says why.
 KERNEL_SOURCES = ("tair_kvcache_amd/csrc/kvcm_copy.hip", "tair_kvcache_amd/csrc/kvcm_hash.hip",
                   "tair_kvcache_amd/csrc/kvcm_internal.h")
-MEASURED_TRAFFIC = {"sources_sha256": "72a535e858f36b02", "unique_blocks": 12416, "gather": 52076667576,
-                    "scatter": 52076193025, "hash_saturated": 571031008}
+MEASURED_TRAFFIC = {"sources_sha256": "72a535e858f36b02", "unique_blocks": 12416, "gather": 52076672905,
+                    "scatter": 52076198457, "hash_saturated": 571029905}
 
 # Llama-3-8B KV layout: the configuration the headline metric is quoted on
 LAYERS, KV_HEADS, HEAD_DIM, ITEMSIZE = 32, 8, 128, 2
@@ -600,7 +600,26 @@ def main():
     # hand-over from the 8 ms load kernel before it
     ms_hash_b2b = gpu_ms(torch, hash_once, 20)
     ms_hash_cold = cold_ms(torch, hash_once, device)
-    del sat_tokens, sat_keys
+    # ApplyPrefixHash (kv_cache_manager/optimizer/trace_converter/trace_util.cc:47-56) on as many chains: the same
+    # 16 384 x 4096 values taken as digests, a key after every step (as many bytes written as read)
+    del sat_keys
+    chain_keys = torch.empty(sat_R * TOKENS_PER_REQ, dtype=torch.int64, device=device)
+    chain_args = (sat_tokens.data_ptr(), sat_toff.data_ptr(), sat_R, chain_keys.data_ptr(),
+                  torch.cuda.current_stream().cuda_stream)
+
+    def chain_once():
+        rc = _lib.lib().kvcm_hip_prefix_chain(*chain_args)
+        if rc != 0:
+            raise SystemExit(f"bench.py: kvcm_hip_prefix_chain failed with code {rc}")
+
+    ms_chain = gpu_ms(torch, chain_once, 5, warm=2)
+    chain_bytes = 2 * sat_R * TOKENS_PER_REQ * 8 + (sat_R + 1) * 8
+    prefix_chain = {"chains": sat_R, "digests_per_chain": TOKENS_PER_REQ, "ms_per_launch": round(ms_chain, 4),
+                    "keys_per_s": round(chain_keys.numel() / (ms_chain * 1e-3)),
+                    "algorithmic_bytes_per_launch": chain_bytes,
+                    "GBps": round(chain_bytes / (ms_chain * 1e-3) / 1e9, 1),
+                    "frac_of_hbm_peak": round(chain_bytes / (ms_chain * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+    del sat_tokens, chain_keys
 
     digest = kernel_sources_digest()
     traffic_ok = digest == MEASURED_TRAFFIC["sources_sha256"]
@@ -668,6 +687,7 @@ def main():
         "verified_against_oracle": verified,
         "roofline": dominant,
         "roofline_hash_saturated": roof_hash,
+        "prefix_chain_saturated": prefix_chain,
         "roofline_save": roof_g, "roofline_load": roof_s,
         "reference_signature": reference_signature,
         "kernel_sources_sha256": digest,
