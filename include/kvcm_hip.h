@@ -12,9 +12,13 @@
  *   - every pointer whose name starts with d_ is DEVICE memory, readable/writable by kernels on the
  *     current HIP device; everything else is host memory;
  *   - all kvcm_hip_* entry points are asynchronous on `stream` (a hipStream_t passed as void*; NULL = null stream),
- *     never synchronise, never allocate, never switch device, and keep no global mutable state, so they
- *     can be called concurrently from many host threads (the reference calls its kernels from a
- *     32-thread pool: kv_cache_manager/py_connector/vllm/data_transfer.py:80-93);
+ *     never synchronise, never allocate and never switch device. With ONE exception they keep no mutable state
+ *     inside the library, so they can be called concurrently from many host threads (the reference calls its
+ *     kernels from a 32-thread pool: kv_cache_manager/py_connector/vllm/data_transfer.py:80-93). The exception is
+ *     kvcm_hip_first_occurrence_static: its table is a device array owned by the library, one per GPU, shared by
+ *     every call on that GPU -- calls that overlap on one GPU race (see its prototype);
+ *   - the library reads no environment variable per call and exports no switch: the one tuning knob,
+ *     KVCM_COPY_XCD_REMAP, is read once when the first copy is launched;
  *   - device buffers passed in must stay alive until `stream` has executed the call;
  *   - the kvcm_file_store_* family at the end is host-side file I/O: it blocks, and it owns streams and pinned
  *     buffers between create and destroy;
@@ -40,6 +44,7 @@ typedef void *kvcm_stream_t;
 #define KVCM_ERR_ALIGNMENT (-2)   /* an address or stride is not aligned as the entry point requires */
 #define KVCM_ERR_TOO_LARGE (-3)   /* a size exceeds what the launch geometry can express */
 #define KVCM_ERR_IO (-4)          /* a file could not be created, opened, grown, read or written */
+#define KVCM_ERR_OUT_OF_RANGE (-5) /* an index in a HOST index list names a slot beyond the size the caller stated */
 
 /* Library version: major*10000 + minor*100 + patch. */
 int32_t kvcm_hip_version(void);
@@ -128,6 +133,35 @@ int32_t kvcm_hip_batch_scatter(const void *const *d_ptr_table, int32_t P, const 
                                int64_t staging_block_stride_bytes, const int32_t *d_token_idx,
                                const int32_t *d_staging_idx, int32_t B, int32_t T, int64_t row_bytes,
                                int32_t max_workgroups, kvcm_stream_t stream);
+
+/*
+ * gather / scatter with the index lists in HOST memory -- the form in which the reference's operators receive them
+ * (Python lists, turned into tensors and uploaded per call:
+ * kv_cache_manager/py_connector/kernel/batch_gather_scatter_helper.py:116-121,223-228; call sites
+ * kv_cache_manager/py_connector/vllm/data_transfer.py:139-146,206-213). Same results as kvcm_hip_batch_gather /
+ * kvcm_hip_batch_scatter on the uploaded lists. Nothing is uploaded and nothing is allocated: the lists are walked once
+ * on the calling thread and travel to the kernel inside its argument block, so they may be freed or overwritten as soon
+ * as the call returns, and the call can be captured into a HIP graph. During that walk
+ *   - every token slot is checked against pool_slots (the number of token slots of each pool array; 0 = not checked)
+ *     and every staging slot against staging_slots (0 = only "not negative" is checked): KVCM_ERR_OUT_OF_RANGE, and
+ *     nothing is launched, when one is out of range. A NEGATIVE token slot is not an error: that row is skipped, as in
+ *     the device-index entry points;
+ *   - when the T slots of every work block turn out to be runs of r consecutive slots (r = T whenever a manager block
+ *     is a whole number of engine blocks) the launch takes the block-table form below with run_tokens = r.
+ * A call is split into several launches when its tables exceed one argument block (3328 bytes: 416 blocks per launch
+ * in block-table form, 48 with 16 unrelated slots per block). KVCM_ERR_TOO_LARGE when a single block has more than
+ * 831 runs: upload the list and use the device-index entry points then. h_staging_idx may be NULL (slot b).
+ */
+int32_t kvcm_hip_batch_gather_host_idx(const void *const *d_ptr_table, int32_t P, void *d_staging,
+                                       int64_t staging_block_stride_bytes, int64_t staging_slots,
+                                       const int32_t *h_token_idx, const int32_t *h_staging_idx, int32_t B, int32_t T,
+                                       int64_t row_bytes, int64_t pool_slots, int32_t max_workgroups,
+                                       kvcm_stream_t stream);
+int32_t kvcm_hip_batch_scatter_host_idx(const void *const *d_ptr_table, int32_t P, const void *d_staging,
+                                        int64_t staging_block_stride_bytes, int64_t staging_slots,
+                                        const int32_t *h_token_idx, const int32_t *h_staging_idx, int32_t B, int32_t T,
+                                        int64_t row_bytes, int64_t pool_slots, int32_t max_workgroups,
+                                        kvcm_stream_t stream);
 
 /*
  * Block-table fast path: the T tokens of work block b are T / run_tokens runs of `run_tokens`

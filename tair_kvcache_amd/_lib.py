@@ -27,6 +27,7 @@ ERR_INVALID_ARG = -1
 ERR_ALIGNMENT = -2
 ERR_TOO_LARGE = -3
 ERR_IO = -4
+ERR_OUT_OF_RANGE = -5
 
 i32, i64, vp, sz = C.c_int32, C.c_int64, C.c_void_p, C.c_size_t
 
@@ -57,6 +58,8 @@ SIGNATURES = {
     "kvcm_hip_sha256_first8_be": (i32, [vp, vp, i32, vp, vp]),
     "kvcm_hip_batch_gather": (i32, [vp, i32, vp, i64, vp, vp, i32, i32, i64, i32, vp]),
     "kvcm_hip_batch_scatter": (i32, [vp, i32, vp, i64, vp, vp, i32, i32, i64, i32, vp]),
+    "kvcm_hip_batch_gather_host_idx": (i32, [vp, i32, vp, i64, i64, vp, vp, i32, i32, i64, i64, i32, vp]),
+    "kvcm_hip_batch_scatter_host_idx": (i32, [vp, i32, vp, i64, i64, vp, vp, i32, i32, i64, i64, i32, vp]),
     "kvcm_hip_paged_gather": (i32, [vp, i32, vp, i64, vp, i32, vp, i32, i32, i64, i32, vp]),
     "kvcm_hip_paged_scatter": (i32, [vp, i32, vp, i64, vp, i32, vp, i32, i32, i64, i32, vp]),
     "kvcm_hip_gather_ex": (i32, [C.POINTER(CopyDesc), vp]),

@@ -16,6 +16,7 @@ is whatever object offers send(bytes) (TpCoordinatorClient, kv_cache_manager/py_
 import math
 import threading
 import time
+from array import array
 from concurrent.futures import ThreadPoolExecutor
 from dataclasses import dataclass
 from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
@@ -192,6 +193,7 @@ class DataTransferManager:
         # object, its callbacks and its result plumbing can be built and tested where there is no GPU
         self._stream_lock = threading.Lock()
         self._streams: Dict[str, Any] = {}
+        self._slot_buffer_cache: Dict[int, Any] = {}
 
     def _stream(self, which: str):
         s = self._streams.get(which)
@@ -223,23 +225,34 @@ class DataTransferManager:
         if isinstance(block_token_indices, torch.Tensor):
             return block_token_indices
         if len(block_token_indices) > 0 and isinstance(block_token_indices[0], (list, tuple)):
-            return [t for row in block_token_indices for t in row]
+            flat = array("i")  # what the operator would turn a flat list into anyway, built row by row
+            try:
+                for row in block_token_indices:
+                    flat.extend(row)
+            except (TypeError, OverflowError) as e:
+                raise ValueError(f"block_token_indices must hold ints that fit 32 bits: {e}") from e
+            return flat
         return block_token_indices
 
     def _slot_buffers(self, slot_indices):
-        on_gpu = self._copy_buffer_allocator.device.type != "cpu"
-        mem = self._cm.MemoryType.GPU if on_gpu else self._cm.MemoryType.CPU
-        buffers = []
-        for slot in self._copy_buffer_allocator.get_buffer_by_idx(slot_indices):
-            iov = self._cm.Iov()
-            iov.type = mem
-            iov.base = slot.data_ptr()
-            iov.size = slot.numel() * slot.element_size()
-            iov.ignore = False
-            buf = self._cm.BlockBuffer()
-            buf.iovs = [iov]
-            buffers.append(buf)
-        return buffers
+        """One BlockBuffer of one Iov per staging slot (data_transfer.py:124-135,218-229). A slot's address and size
+        never change, so its buffer object is built once and handed out again: building 128 Iov and BlockBuffer objects
+        per task costs more interpreter time than everything else a task does on the host."""
+        cache = self._slot_buffer_cache
+        missing = [i for i in slot_indices if i not in cache]
+        if missing:
+            on_gpu = self._copy_buffer_allocator.device.type != "cpu"
+            mem = self._cm.MemoryType.GPU if on_gpu else self._cm.MemoryType.CPU
+            for i, slot in zip(missing, self._copy_buffer_allocator.get_buffer_by_idx(missing)):
+                iov = self._cm.Iov()
+                iov.type = mem
+                iov.base = slot.data_ptr()
+                iov.size = slot.numel() * slot.element_size()
+                iov.ignore = False
+                buf = self._cm.BlockBuffer()
+                buf.iovs = [iov]
+                cache[i] = buf  # a dict store is atomic; two threads that build the same slot build equal objects
+        return [cache[i] for i in slot_indices]
 
     def load_task(self, multi_result: MultiResult, task_idx: int, remote_uris: List[str], block_token_indices):
         ok = self._cm.ClientErrorCode.ER_OK
@@ -251,7 +264,8 @@ class DataTransferManager:
                     batch_gather_scatter_helper.batch_scatter_kv_caches(
                         self._kvcache_info.all_kvcache_ptr_tensor_gpu, self._copy_buffer_allocator._raw_buffer,
                         self._flat_indices(block_token_indices), slots, self._manager_block_size,
-                        self._kvcache_info.per_token_per_layer_dim_size)
+                        self._kvcache_info.per_token_per_layer_dim_size,
+                        pool_token_slots=self._kvcache_info.local_token_num)
                     done = torch.cuda.Event()
                     done.record(self._load_stream)
                 done.synchronize()
@@ -308,7 +322,8 @@ class DataTransferManager:
                 batch_gather_scatter_helper.batch_gather_kv_caches(
                     self._kvcache_info.all_kvcache_ptr_tensor_gpu, self._copy_buffer_allocator._raw_buffer,
                     self._flat_indices(block_token_indices), slots, self._manager_block_size,
-                    self._kvcache_info.per_token_per_layer_dim_size)
+                    self._kvcache_info.per_token_per_layer_dim_size,
+                    pool_token_slots=self._kvcache_info.local_token_num)
                 done = torch.cuda.Event()
                 done.record(self._save_stream)
             done.synchronize()

@@ -181,15 +181,33 @@ __device__ __forceinline__ void store_chunk16(unsigned char *p, u32x4 v) {
 //   kRunPerThread anything else: the run number is a multiply-shift division per thread and the slot a vector load.
 enum RunMode { kRunPerThread = 0, kRunPerWave = 1, kRunPerGroup = 2 };
 
-template <int CS, bool SCATTER, bool UNI_TILE, int RUN>
-__global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
-                                                             // read-only tables, never written by this kernel:
-                                                             // __restrict__ lets uniform reads become scalar loads
-                                                             const void *const *__restrict__ ptr_table,
-                                                             const void *const *__restrict__ trailer_table,
-                                                             const int32_t *__restrict__ run_start,
-                                                             const int32_t *__restrict__ staging_idx,
-                                                             const int32_t *__restrict__ trailer_idx) {
+// Where a launch finds its index tables. PtrIdx: two arrays in device memory (every entry point that takes d_ pointers).
+// KernargIdx: the tables travel INSIDE the kernel's argument block, run starts first, staging slots behind them -- the
+// form behind the entry points that take host index lists: nothing is uploaded, nothing has to outlive the call, and a
+// uniform read of the table is a scalar load from the argument segment like any other kernel argument.
+constexpr int kEmbedInts = 832;  // 3328 bytes of the 4 KiB a kernel's argument block may have
+struct EmbeddedIdx {
+    int32_t v[kEmbedInts];
+};
+struct PtrIdx {
+    const int32_t *run_start;
+    const int32_t *staging_idx;
+    __device__ __forceinline__ int32_t run(int64_t i) const { return run_start[i]; }
+    __device__ __forceinline__ int64_t slot(uint32_t b) const {
+        return staging_idx ? staging_idx[b] : static_cast<int64_t>(b);
+    }
+};
+struct KernargIdx {
+    const EmbeddedIdx &e;
+    uint32_t staging_first;  // index of the first staging slot inside e.v
+    __device__ __forceinline__ int32_t run(int64_t i) const { return e.v[i]; }
+    __device__ __forceinline__ int64_t slot(uint32_t b) const { return e.v[staging_first + b]; }
+};
+
+template <int CS, bool SCATTER, bool UNI_TILE, int RUN, typename Idx>
+__device__ __forceinline__ void copy_span_body(const CopyArgs &a, const void *const *__restrict__ ptr_table,
+                                               const void *const *__restrict__ trailer_table, const Idx &idx,
+                                               const int32_t *__restrict__ trailer_idx) {
     using V = typename Chunk<CS>::V;
 
     // Consecutive workgroup ids land on consecutive XCDs (8 per device, one L2 each). With the remap every XCD
@@ -205,7 +223,7 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
     for (uint32_t unit = first; unit < a.n_units; unit += gridDim.x) {
         const uint32_t b = fast_div(unit, a.div_units);
         const uint32_t span = unit - b * a.units_per_block;
-        const int32_t *runs_b = run_start + static_cast<int64_t>(b) * a.runs;
+        const int64_t runs_b = static_cast<int64_t>(b) * a.runs;  // index of the block's first run
         // workgroup-uniform part: the three table reads below are independent scalar loads in the UNI_* forms
         const uint32_t g_first = span * kSpan;
         const uint32_t p_first = fast_div(g_first, a.div_tile);
@@ -215,11 +233,11 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
         int64_t slot_shared = 0;
         uint32_t r_shared = r_first;
         if (RUN == kRunPerGroup) {
-            slot_shared = runs_b[r_first];
+            slot_shared = idx.run(runs_b + r_first);
         } else if (RUN == kRunPerWave) {
             // one chunk per thread: a wave's 64 chunks start at a multiple of 64 and lie inside one run
             r_shared = __builtin_amdgcn_readfirstlane(fast_div(cc_first + (threadIdx.x & ~63u), a.div_run));
-            slot_shared = runs_b[r_shared];
+            slot_shared = idx.run(runs_b + r_shared);
         }
         const void *pool_first = UNI_TILE ? ptr_table[entry_first] : nullptr;
         // the span that starts a tile also moves the tile's trailer: its table entries are workgroup-uniform too
@@ -229,7 +247,7 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
             trailer_idx_first = trailer_idx[b];
             trailer_base_first = trailer_table[p_first];
         }
-        const int64_t slot_b = staging_idx ? staging_idx[b] : static_cast<int64_t>(b);
+        const int64_t slot_b = idx.slot(b);
         unsigned char *block = a.staging + slot_b * a.block_stride;
 
         V v[kCPT];
@@ -248,7 +266,7 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
                 const uint32_t cc = UNI_TILE ? cc_first + in_span : g - p * a.chunks_per_tile;
                 const uint32_t r = RUN != kRunPerThread ? r_shared : fast_div(cc, a.div_run);
                 const uint32_t off = cc - r * a.chunks_per_run;
-                const int64_t slot = RUN != kRunPerThread ? slot_shared : static_cast<int64_t>(runs_b[r]);
+                const int64_t slot = RUN != kRunPerThread ? slot_shared : static_cast<int64_t>(idx.run(runs_b + r));
                 unsigned char *tile = block + static_cast<int64_t>(p) * a.tile_stride;
                 if (slot >= 0 && slot < limit) {
                     const uint32_t entry = UNI_TILE ? entry_first : fast_div(p, a.div_entry);
@@ -345,6 +363,28 @@ __global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
     }
 }
 
+template <int CS, bool SCATTER, bool UNI_TILE, int RUN>
+__global__ __launch_bounds__(kThreads) void copy_span_kernel(const CopyArgs a,
+                                                             // read-only tables, never written by this kernel:
+                                                             // __restrict__ lets uniform reads become scalar loads
+                                                             const void *const *__restrict__ ptr_table,
+                                                             const void *const *__restrict__ trailer_table,
+                                                             const int32_t *__restrict__ run_start,
+                                                             const int32_t *__restrict__ staging_idx,
+                                                             const int32_t *__restrict__ trailer_idx) {
+    copy_span_body<CS, SCATTER, UNI_TILE, RUN>(a, ptr_table, trailer_table, PtrIdx{run_start, staging_idx}, trailer_idx);
+}
+
+// The same kernel with its index tables in the argument block (host index lists).
+template <int CS, bool SCATTER, bool UNI_TILE, int RUN>
+__global__ __launch_bounds__(kThreads) void copy_span_kernarg_kernel(const EmbeddedIdx emb, const CopyArgs a,
+                                                                     uint32_t staging_first,
+                                                                     const void *const *__restrict__ ptr_table,
+                                                                     const void *const *__restrict__ trailer_table,
+                                                                     const int32_t *__restrict__ trailer_idx) {
+    copy_span_body<CS, SCATTER, UNI_TILE, RUN>(a, ptr_table, trailer_table, KernargIdx{emb, staging_first}, trailer_idx);
+}
+
 // out[b][i] = block_ids[(m_b*T_mgr + i) / T_eng] * T_eng + (m_b*T_mgr + i) % T_eng
 // (kv_cache_manager/py_connector/vllm/v1_connector.py:308-320).
 __global__ __launch_bounds__(256) void blocks_idx_kernel(const int32_t *mgr, int32_t B, const int32_t *local_ids,
@@ -382,9 +422,20 @@ int32_t align_class(uint64_t bits) {
     return 1;
 }
 
+// emb != nullptr: the index tables are *emb (copied into the kernel's argument block by the launch), run starts from
+// entry 0, staging slots from entry `staging_first`; the descriptor's d_run_start / d_staging_idx are not looked at.
 template <int CS, bool UNI_TILE, int RUN>
-void launch_span(const CopyArgs &a, const kvcm_copy_desc *d, bool scatter, uint32_t grid, hipStream_t stream) {
-    if (scatter) {
+void launch_span(const CopyArgs &a, const kvcm_copy_desc *d, bool scatter, uint32_t grid, hipStream_t stream,
+                 const EmbeddedIdx *emb, uint32_t staging_first) {
+    if (emb) {
+        if (scatter) {
+            hipLaunchKernelGGL((copy_span_kernarg_kernel<CS, true, UNI_TILE, RUN>), dim3(grid), dim3(kThreads), 0,
+                               stream, *emb, a, staging_first, d->d_ptr_table, d->d_trailer_ptr_table, d->d_trailer_idx);
+        } else {
+            hipLaunchKernelGGL((copy_span_kernarg_kernel<CS, false, UNI_TILE, RUN>), dim3(grid), dim3(kThreads), 0,
+                               stream, *emb, a, staging_first, d->d_ptr_table, d->d_trailer_ptr_table, d->d_trailer_idx);
+        }
+    } else if (scatter) {
         hipLaunchKernelGGL((copy_span_kernel<CS, true, UNI_TILE, RUN>), dim3(grid), dim3(kThreads), 0, stream, a,
                            d->d_ptr_table, d->d_trailer_ptr_table, d->d_run_start, d->d_staging_idx, d->d_trailer_idx);
     } else {
@@ -393,7 +444,8 @@ void launch_span(const CopyArgs &a, const kvcm_copy_desc *d, bool scatter, uint3
     }
 }
 
-int32_t launch_copy(const kvcm_copy_desc *d, bool scatter, hipStream_t stream) {
+int32_t launch_copy(const kvcm_copy_desc *d, bool scatter, hipStream_t stream, const EmbeddedIdx *emb = nullptr,
+                    uint32_t staging_first = 0) {
     if (!d) {
         return KVCM_ERR_INVALID_ARG;
     }
@@ -412,7 +464,7 @@ int32_t launch_copy(const kvcm_copy_desc *d, bool scatter, hipStream_t stream) {
     if (d->B == 0) {
         return KVCM_OK;
     }
-    if (!d->d_ptr_table || !d->d_staging || !d->d_run_start) {
+    if (!d->d_ptr_table || !d->d_staging || (!emb && !d->d_run_start)) {
         return KVCM_ERR_INVALID_ARG;
     }
     if (d->trailer_bytes > 0 && (!d->d_trailer_ptr_table || !d->d_trailer_idx)) {
@@ -465,17 +517,17 @@ int32_t launch_copy(const kvcm_copy_desc *d, bool scatter, hipStream_t stream) {
     a.staging_on_line_grid = ((reinterpret_cast<uint64_t>(d->d_staging) | static_cast<uint64_t>(a.block_stride) |
                                static_cast<uint64_t>(a.tile_stride)) & 127u) == 0;
     if (cs == 16 && uni_tile && a.chunks_per_run % kSpan == 0) {
-        launch_span<16, true, kRunPerGroup>(a, d, scatter, g32, stream);
+        launch_span<16, true, kRunPerGroup>(a, d, scatter, g32, stream, emb, staging_first);
     } else if (cs == 16 && uni_tile && kCPT == 1 && a.chunks_per_run % 64 == 0) {
-        launch_span<16, true, kRunPerWave>(a, d, scatter, g32, stream);
+        launch_span<16, true, kRunPerWave>(a, d, scatter, g32, stream, emb, staging_first);
     } else if (cs == 16 && uni_tile) {
-        launch_span<16, true, kRunPerThread>(a, d, scatter, g32, stream);
+        launch_span<16, true, kRunPerThread>(a, d, scatter, g32, stream, emb, staging_first);
     } else if (cs == 16) {
-        launch_span<16, false, kRunPerThread>(a, d, scatter, g32, stream);
+        launch_span<16, false, kRunPerThread>(a, d, scatter, g32, stream, emb, staging_first);
     } else if (cs == 4) {
-        launch_span<4, false, kRunPerThread>(a, d, scatter, g32, stream);
+        launch_span<4, false, kRunPerThread>(a, d, scatter, g32, stream, emb, staging_first);
     } else {
-        launch_span<1, false, kRunPerThread>(a, d, scatter, g32, stream);
+        launch_span<1, false, kRunPerThread>(a, d, scatter, g32, stream, emb, staging_first);
     }
     return launch_status();
 }
@@ -500,6 +552,82 @@ kvcm_copy_desc flat_desc(const void *const *d_ptr_table, int32_t P, void *d_stag
     d.row_bytes = row_bytes;
     d.max_workgroups = max_workgroups;
     return d;
+}
+
+// Host index lists -> launches whose tables ride in the argument block. One pass over the lists does what the callers
+// of the device-index entry points do on their side: range checks, and the discovery that the T slots of every block are
+// runs of r consecutive slots (r = T when a manager block is k engine blocks: the block-table form, a sixteenth of the
+// index reads and workgroup-uniform address arithmetic).
+int32_t launch_copy_host_idx(const void *const *d_ptr_table, int32_t P, void *d_staging, int64_t block_stride,
+                             int64_t staging_slots, const int32_t *h_token_idx, const int32_t *h_staging_idx, int32_t B,
+                             int32_t T, int64_t row_bytes, int64_t pool_slots, int32_t max_workgroups, bool scatter,
+                             hipStream_t stream) {
+    if (B < 0 || T <= 0 || P <= 0 || row_bytes <= 0 || staging_slots < 0 || pool_slots < 0) {
+        return KVCM_ERR_INVALID_ARG;
+    }
+    if (B == 0) {
+        return KVCM_OK;
+    }
+    if (!h_token_idx || !d_ptr_table || !d_staging) {
+        return KVCM_ERR_INVALID_ARG;
+    }
+    // r = gcd(T, every position inside a block where the slot is not its predecessor's + 1)
+    const auto gcd = [](uint32_t x, uint32_t y) {
+        while (y) {
+            const uint32_t t = x % y;
+            x = y;
+            y = t;
+        }
+        return x;
+    };
+    uint32_t r = static_cast<uint32_t>(T);
+    const int64_t pool_limit = pool_slots > 0 ? pool_slots : (int64_t{1} << 31);
+    for (int32_t b = 0; b < B; ++b) {
+        const int32_t *row = h_token_idx + static_cast<int64_t>(b) * T;
+        if (row[0] >= pool_limit) {
+            return KVCM_ERR_OUT_OF_RANGE;
+        }
+        for (int32_t j = 1; j < T; ++j) {
+            if (row[j] >= pool_limit) {
+                return KVCM_ERR_OUT_OF_RANGE;
+            }
+            // a negative slot means "skip this row": it never joins a run, so that nothing but that row is skipped
+            if (r > 1 && (row[j - 1] < 0 || row[j] != row[j - 1] + 1)) {
+                r = gcd(r, static_cast<uint32_t>(j));
+            }
+        }
+        if (h_staging_idx) {
+            const int64_t sb = h_staging_idx[b];
+            if (sb < 0 || (staging_slots > 0 && sb >= staging_slots)) {
+                return KVCM_ERR_OUT_OF_RANGE;
+            }
+        } else if (staging_slots > 0 && b >= staging_slots) {
+            return KVCM_ERR_OUT_OF_RANGE;
+        }
+    }
+    const int32_t runs = T / static_cast<int32_t>(r);
+    if (runs + 1 > kEmbedInts) {
+        return KVCM_ERR_TOO_LARGE;  // one block's table does not fit an argument block: upload it instead
+    }
+    const int32_t per_launch = kEmbedInts / (runs + 1);
+    EmbeddedIdx emb;
+    for (int32_t b0 = 0; b0 < B; b0 += per_launch) {
+        const int32_t nb = B - b0 < per_launch ? B - b0 : per_launch;
+        for (int32_t i = 0; i < nb; ++i) {
+            const int32_t *row = h_token_idx + static_cast<int64_t>(b0 + i) * T;
+            for (int32_t k = 0; k < runs; ++k) {
+                emb.v[i * runs + k] = row[k * static_cast<int32_t>(r)];
+            }
+            emb.v[nb * runs + i] = h_staging_idx ? h_staging_idx[b0 + i] : b0 + i;
+        }
+        kvcm_copy_desc d = flat_desc(d_ptr_table, P, d_staging, block_stride, nullptr, static_cast<int32_t>(r), nullptr,
+                                     nb, T, row_bytes, max_workgroups);
+        const int32_t rc = launch_copy(&d, scatter, stream, &emb, static_cast<uint32_t>(nb * runs));
+        if (rc != KVCM_OK) {
+            return rc;
+        }
+    }
+    return KVCM_OK;
 }
 
 }  // namespace
@@ -532,6 +660,26 @@ int32_t kvcm_hip_batch_scatter(const void *const *d_ptr_table, int32_t P, const 
     kvcm_copy_desc d = kvcm::flat_desc(d_ptr_table, P, const_cast<void *>(d_staging), staging_block_stride_bytes,
                                        d_token_idx, 1, d_staging_idx, B, T, row_bytes, max_workgroups);
     return kvcm::launch_copy(&d, true, static_cast<hipStream_t>(stream));
+}
+
+int32_t kvcm_hip_batch_gather_host_idx(const void *const *d_ptr_table, int32_t P, void *d_staging,
+                                       int64_t staging_block_stride_bytes, int64_t staging_slots,
+                                       const int32_t *h_token_idx, const int32_t *h_staging_idx, int32_t B, int32_t T,
+                                       int64_t row_bytes, int64_t pool_slots, int32_t max_workgroups,
+                                       kvcm_stream_t stream) {
+    return kvcm::launch_copy_host_idx(d_ptr_table, P, d_staging, staging_block_stride_bytes, staging_slots, h_token_idx,
+                                      h_staging_idx, B, T, row_bytes, pool_slots, max_workgroups, false,
+                                      static_cast<hipStream_t>(stream));
+}
+
+int32_t kvcm_hip_batch_scatter_host_idx(const void *const *d_ptr_table, int32_t P, const void *d_staging,
+                                        int64_t staging_block_stride_bytes, int64_t staging_slots,
+                                        const int32_t *h_token_idx, const int32_t *h_staging_idx, int32_t B, int32_t T,
+                                        int64_t row_bytes, int64_t pool_slots, int32_t max_workgroups,
+                                        kvcm_stream_t stream) {
+    return kvcm::launch_copy_host_idx(d_ptr_table, P, const_cast<void *>(d_staging), staging_block_stride_bytes,
+                                      staging_slots, h_token_idx, h_staging_idx, B, T, row_bytes, pool_slots,
+                                      max_workgroups, true, static_cast<hipStream_t>(stream));
 }
 
 int32_t kvcm_hip_paged_gather(const void *const *d_ptr_table, int32_t P, void *d_staging,

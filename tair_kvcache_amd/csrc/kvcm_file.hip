@@ -117,6 +117,10 @@ struct kvcm_file_store {
     std::condition_variable lane_freed;
     std::vector<kvcm::Lane *> idle;
     int lanes_alive = 0;
+    // puts and gets between entry and return, under `mu`: what kvcm_file_store_destroy waits for before it touches
+    // the helper threads or the lanes
+    int calls_running = 0;
+    std::condition_variable calls_done;
 
     // Helper threads for big reads: started on first need, at most io_threads - 1, alive until the store is destroyed
     // (a thread's first HIP call costs far more than a 256 MiB read, so they are not started per call).
@@ -129,12 +133,18 @@ struct kvcm_file_store {
     std::atomic<int> transfers_in_flight{0};
 
     void submit(std::function<void()> job) {
-        std::lock_guard<std::mutex> lock(pool_mu);
-        pool_jobs.push_back(std::move(job));
-        if (pool_idle == 0 && static_cast<int32_t>(pool.size()) < io_threads - 1) {
-            pool.emplace_back([this] { pool_loop(); });
+        {
+            std::lock_guard<std::mutex> lock(pool_mu);
+            if (!pool_stop) {
+                pool_jobs.push_back(std::move(job));
+                if (pool_idle == 0 && static_cast<int32_t>(pool.size()) < io_threads - 1) {
+                    pool.emplace_back([this] { pool_loop(); });
+                }
+                pool_wake.notify_one();
+                return;
+            }
         }
-        pool_wake.notify_one();
+        job();  // the helper threads are being joined: nobody would take the job, so the caller does it itself
     }
 
     void pool_loop() {
@@ -233,6 +243,23 @@ struct kvcm_file_store {
 
 namespace kvcm {
 namespace {
+
+// Marks a put or get as running from its first look at the store to its return.
+struct CallGuard {
+    kvcm_file_store *store;
+    explicit CallGuard(kvcm_file_store *s) : store(s) {
+        std::lock_guard<std::mutex> lock(store->mu);
+        store->calls_running++;
+    }
+    ~CallGuard() {
+        std::lock_guard<std::mutex> lock(store->mu);
+        if (--store->calls_running == 0) {
+            store->calls_done.notify_all();
+        }
+    }
+    CallGuard(const CallGuard &) = delete;
+    CallGuard &operator=(const CallGuard &) = delete;
+};
 
 // Validation and layout shared by Put and Get (local_file_sdk.cc:197-252, 317-359): returns the byte ranges to
 // move, merged where both sides are contiguous. `limit` is the size no iov may reach beyond.
@@ -441,10 +468,17 @@ void kvcm_file_store_destroy(kvcm_file_store *store) {
     if (!store) {
         return;
     }
+    {
+        // Puts and gets that other threads are still inside of finish first: they may yet hand work to the helper
+        // threads and take lanes. (A call that has not reached its first line when this wait ends is the caller's
+        // bug: no call may start once destruction has begun.)
+        std::unique_lock<std::mutex> lock(store->mu);
+        store->calls_done.wait(lock, [store] { return store->calls_running == 0; });
+    }
     store->stop_pool();
     {
-        // a put or get that is still running holds its lane: wait until every lane is back before freeing them
         std::unique_lock<std::mutex> lock(store->mu);
+        // every lane is back by now (a call returns its lanes before it ends); the wait is a second line of defence
         store->lane_freed.wait(lock, [store] { return static_cast<int>(store->idle.size()) == store->lanes_alive; });
         for (kvcm::Lane *lane : store->idle) {
             kvcm_file_store::destroy(lane);
@@ -460,6 +494,7 @@ int32_t kvcm_file_store_put(kvcm_file_store *store, const char *path, const uint
     if (!store || !path || !*path || n_blocks <= 0 || !blkids || !sizes || !iov_counts) {
         return KVCM_ERR_INVALID_ARG;
     }
+    kvcm::CallGuard running(store);
     const uint64_t bsz = static_cast<uint64_t>(store->byte_size_per_block);
     uint64_t required = 0;
     for (int32_t b = 0; b < n_blocks; b++) {
@@ -510,6 +545,7 @@ int32_t kvcm_file_store_get(kvcm_file_store *store, const char *path, const uint
     if (!store || !path || !*path || n_blocks <= 0 || !blkids || !sizes || !iov_counts) {
         return KVCM_ERR_INVALID_ARG;
     }
+    kvcm::CallGuard running(store);
     int fd = open(path, O_RDONLY);
     if (fd < 0) {
         return KVCM_ERR_IO;

@@ -21,8 +21,7 @@
 // dependent-instruction latency of the chain wave, which no amount of bandwidth removes.
 #include "kvcm_internal.h"
 
-#include <atomic>
-#include <cstdlib>
+#include <climits>
 
 namespace kvcm {
 namespace {
@@ -751,13 +750,13 @@ __global__ __launch_bounds__(256) void iov_crc32_kernel(const kvcm_iov_device *_
     out[i] = ~crc;
 }
 
-// Test hook: non-zero makes every launch take the loader path that a workgroup spanning >= 4 GiB of tokens would take.
-// Starts from the environment variable KVCM_HASH_FORCE_GLOBAL_LOADS (read once, when the library is loaded) and is
-// switched by kvcm_test_hook_hash_force_global_loads, which no header declares.
-std::atomic<int32_t> g_force_global_loads{[] {
-    const char *fg = std::getenv("KVCM_HASH_FORCE_GLOBAL_LOADS");
-    return (fg && fg[0] == '1') ? 1 : 0;
-}()};
+// Non-zero makes every launch take the loader path that a workgroup spanning >= 4 GiB of tokens would take. A
+// compile-time matter: the shipped library is built with 0 and has no switch; the parity tests build this file a second
+// time, with KVCM_TEST_FORCE_GENERAL_LOADER=1, into a library of their own.
+#ifndef KVCM_TEST_FORCE_GENERAL_LOADER
+#define KVCM_TEST_FORCE_GENERAL_LOADER 0
+#endif
+constexpr int32_t kForceGeneralLoader = KVCM_TEST_FORCE_GENERAL_LOADER;
 
 // How keys reach memory, by block size, token width and number of requests in the launch (hash_tokens_kernel<.., KS>).
 // Chosen from timings on tokens that are not in the memory-side cache. 16-token blocks, us for requests of 4096 tokens,
@@ -813,7 +812,7 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
         return KVCM_ERR_INVALID_ARG;
     }
     const dim3 grid(static_cast<uint32_t>((static_cast<int64_t>(R) + kReqs - 1) / kReqs));
-    const int32_t force_global = g_force_global_loads.load(std::memory_order_relaxed);
+    const int32_t force_global = kForceGeneralLoader;
 #define KVCM_LAUNCH_HASH(CHUNK, BS)                                                                                  \
     hipLaunchKernelGGL((hash_tokens_kernel<TokT, CHUNK, BS>), grid, dim3(kThreads), 0, stream, d_tokens,            \
                        d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
@@ -878,12 +877,7 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
 
 extern "C" {
 
-int32_t kvcm_hip_version(void) { return 100; }
-
-// For the parity tests only (not part of the C-ABI): returns the previous setting.
-int32_t kvcm_test_hook_hash_force_global_loads(int32_t on) {
-    return kvcm::g_force_global_loads.exchange(on ? 1 : 0, std::memory_order_relaxed);
-}
+int32_t kvcm_hip_version(void) { return 200; }  // 0.2.0: host-index gather/scatter added, test hook gone
 
 const char *kvcm_hip_error_string(int32_t code) {
     switch (code) {
@@ -897,6 +891,8 @@ const char *kvcm_hip_error_string(int32_t code) {
             return "size exceeds the launch geometry";
         case KVCM_ERR_IO:
             return "file input/output error";
+        case KVCM_ERR_OUT_OF_RANGE:
+            return "index out of range";
         default:
             return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown kvcm error";
     }

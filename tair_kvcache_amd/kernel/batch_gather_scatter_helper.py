@@ -3,12 +3,18 @@
 Drop-in for kv_cache_manager/py_connector/kernel/batch_gather_scatter_helper.py:101-136,208-248: same names,
 same positional order, same defaults. Differences a caller can rely on:
   - index arguments may also be int32 tensors (CPU or device); device tensors are used without a copy;
+  - index arguments in host memory (Python lists, CPU tensors) are not uploaded at all: they are walked once on the
+    calling thread -- range checks, and the discovery that a block's slots are consecutive, which turns the launch
+    into the block-table form -- and travel to the kernel inside its argument block (kvcm_hip_batch_*_host_idx);
+  - `pool_token_slots` (keyword only) = token slots per pool array: with it, a token slot beyond the pool raises
+    ValueError before anything is launched (the reference checks nothing; a wild slot is a GPU memory fault);
   - the staging tensor may live in HBM or in pinned host memory;
   - `sm_count` (the reference's 3-program PCIe throttle, :110,:115) is accepted and ignored unless
     SM_COUNT_IS_CAP is set, in which case it caps the number of workgroups;
   - shape mismatches raise ValueError before anything is launched (the reference lets Triton fail).
 The launch is asynchronous on the current torch stream and never synchronises, like the reference's.
 """
+from array import array
 from typing import List, Sequence, Union
 
 import torch
@@ -22,8 +28,7 @@ IndexArg = Union[List[int], Sequence[int], torch.Tensor]
 SM_COUNT_IS_CAP = False
 
 
-def _prepare(kv_caches_ptrs_tensor, staging, block_token_indices, block_indices, num_tokens_per_block,
-             dim_size_per_token_per_layer, run_tokens=1):
+def _geometry(kv_caches_ptrs_tensor, staging, num_tokens_per_block, dim_size_per_token_per_layer, run_tokens=1):
     require_cuda(kv_caches_ptrs_tensor, "kv_caches_ptrs_tensor")
     if kv_caches_ptrs_tensor.dtype != torch.int64 or kv_caches_ptrs_tensor.dim() != 1:
         raise ValueError("kv_caches_ptrs_tensor must be a 1-D int64 tensor of device pointers")
@@ -36,16 +41,23 @@ def _prepare(kv_caches_ptrs_tensor, staging, block_token_indices, block_indices,
     T, D = int(num_tokens_per_block), int(dim_size_per_token_per_layer)
     if T <= 0 or D <= 0 or run_tokens <= 0 or T % run_tokens != 0:
         raise ValueError("num_tokens_per_block and dim_size_per_token_per_layer must be positive")
-    device = kv_caches_ptrs_tensor.device
     P = kv_caches_ptrs_tensor.numel()
     if P == 0:
         raise ValueError("kv_caches_ptrs_tensor is empty")
-    row_bytes = D * staging.element_size()
+    esz = staging.element_size()
+    row_bytes = D * esz
     block_bytes = P * T * row_bytes
-    if staging.numel() == 0 or (staging.numel() * staging.element_size()) % block_bytes != 0:
+    nbytes = staging.numel() * esz
+    if nbytes == 0 or nbytes % block_bytes != 0:
         raise ValueError(
             f"staging tensor of {staging.numel()} elements is not a whole number of [P={P}, T={T}, D={D}] blocks")
-    slots = staging.numel() * staging.element_size() // block_bytes
+    return kv_caches_ptrs_tensor.device, P, T, row_bytes, block_bytes, nbytes // block_bytes
+
+
+def _prepare(kv_caches_ptrs_tensor, staging, block_token_indices, block_indices, num_tokens_per_block,
+             dim_size_per_token_per_layer, run_tokens=1):
+    device, P, T, row_bytes, block_bytes, slots = _geometry(
+        kv_caches_ptrs_tensor, staging, num_tokens_per_block, dim_size_per_token_per_layer, run_tokens)
     sidx = as_device_i32(block_indices, device, "block indices")
     B = sidx.numel()
     tidx = as_device_i32(block_token_indices, device, "block_token_indices")
@@ -56,6 +68,51 @@ def _prepare(kv_caches_ptrs_tensor, staging, block_token_indices, block_indices,
         if min(block_indices) < 0 or max(block_indices) >= slots:
             raise ValueError(f"staging block index out of range [0, {slots})")
     return device, P, T, row_bytes, block_bytes, tidx, sidx, B
+
+
+def _host_i32(values, name):
+    """(address, count, keep-alive) of `values` as int32 in host memory, or None when `values` lives on the GPU.
+    A list goes through array('i'): one C loop over the list, a third of the time of building a tensor from it."""
+    if isinstance(values, torch.Tensor):
+        if values.is_cuda:
+            return None
+        t = values.reshape(-1)
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            t = t.to(torch.int32).contiguous()
+        return t.data_ptr(), t.numel(), t
+    try:
+        a = values if isinstance(values, array) and values.typecode == "i" else array("i", values)
+    except (TypeError, OverflowError) as e:
+        raise ValueError(f"{name} must be a list of ints that fit 32 bits, or an integer tensor: {e}") from e
+    return a.buffer_info()[0], len(a), a
+
+
+def _run(host_fn, device_fn, kv_caches_ptrs_tensor, staging, block_token_indices, block_indices,
+         num_tokens_per_block, dim_size_per_token_per_layer, sm_count, pool_token_slots):
+    """Host index lists take the entry point that carries them in the kernel's argument block; anything on the GPU
+    (or a block of more runs than an argument block holds) takes the device-index entry point."""
+    tok = _host_i32(block_token_indices, "block_token_indices")
+    sl = _host_i32(block_indices, "block indices") if tok is not None else None
+    if tok is not None and sl is not None:
+        device, P, T, row_bytes, block_bytes, slots = _geometry(
+            kv_caches_ptrs_tensor, staging, num_tokens_per_block, dim_size_per_token_per_layer)
+        B = sl[1]
+        if tok[1] != B * T:
+            raise ValueError(f"block_token_indices has {tok[1]} entries, expected {B} blocks x {T}")
+        rc = host_fn(ptr(kv_caches_ptrs_tensor), P, ptr(staging), block_bytes, slots, tok[0], sl[0], B, T, row_bytes,
+                     int(pool_token_slots or 0), _cap(sm_count), stream_handle(device))
+        if rc == _lib.ERR_OUT_OF_RANGE:
+            raise ValueError(f"index out of range: staging slots must lie in [0, {slots}), token slots below "
+                             f"pool_token_slots ({pool_token_slots})")
+        if rc != _lib.ERR_TOO_LARGE:
+            _lib.check(rc, host_fn.__name__)
+            return
+    device, P, T, row_bytes, block_bytes, tidx, sidx, B = _prepare(
+        kv_caches_ptrs_tensor, staging, block_token_indices, block_indices, num_tokens_per_block,
+        dim_size_per_token_per_layer)
+    rc = device_fn(ptr(kv_caches_ptrs_tensor), P, ptr(staging), block_bytes, ptr(tidx), ptr(sidx), B, T, row_bytes,
+                   _cap(sm_count), stream_handle(device))
+    _lib.check(rc, device_fn.__name__)
 
 
 def _cap(sm_count):
@@ -69,14 +126,13 @@ def batch_gather_kv_caches(
         dst_block_indices: IndexArg,  # B staging slots
         num_tokens_per_block: int,
         dim_size_per_token_per_layer: int,
-        sm_count: int = 3):
+        sm_count: int = 3,
+        *, pool_token_slots: int = 0):
     """dst[sb[b], p, t, :] = pool_p[idx[b*T + t], :]  (batch_gather_scatter_helper.py:49-98)."""
-    device, P, T, row_bytes, block_bytes, tidx, sidx, B = _prepare(
-        kv_caches_ptrs_tensor, dst_tensor, block_token_indices, dst_block_indices, num_tokens_per_block,
-        dim_size_per_token_per_layer)
-    rc = lib().kvcm_hip_batch_gather(ptr(kv_caches_ptrs_tensor), P, ptr(dst_tensor), block_bytes, ptr(tidx),
-                                     ptr(sidx), B, T, row_bytes, _cap(sm_count), stream_handle(device))
-    _lib.check(rc, "kvcm_hip_batch_gather")
+    L = lib()
+    _run(L.kvcm_hip_batch_gather_host_idx, L.kvcm_hip_batch_gather, kv_caches_ptrs_tensor, dst_tensor,
+         block_token_indices, dst_block_indices, num_tokens_per_block, dim_size_per_token_per_layer, sm_count,
+         pool_token_slots)
 
 
 def batch_scatter_kv_caches(
@@ -86,16 +142,15 @@ def batch_scatter_kv_caches(
         src_block_indices: IndexArg,
         num_tokens_per_block: int,
         dim_size_per_token_per_layer: int,
-        sm_count: int = 3):
+        sm_count: int = 3,
+        *, pool_token_slots: int = 0):
     """pool_p[idx[b*T + t], :] = src[sb[b], p, t, :]  (batch_gather_scatter_helper.py:155-205).
 
     Two work blocks that name the same pool row race; callers must not pass duplicates."""
-    device, P, T, row_bytes, block_bytes, tidx, sidx, B = _prepare(
-        kv_caches_ptrs_tensor, src_tensor, block_token_indices, src_block_indices, num_tokens_per_block,
-        dim_size_per_token_per_layer)
-    rc = lib().kvcm_hip_batch_scatter(ptr(kv_caches_ptrs_tensor), P, ptr(src_tensor), block_bytes, ptr(tidx),
-                                      ptr(sidx), B, T, row_bytes, _cap(sm_count), stream_handle(device))
-    _lib.check(rc, "kvcm_hip_batch_scatter")
+    L = lib()
+    _run(L.kvcm_hip_batch_scatter_host_idx, L.kvcm_hip_batch_scatter, kv_caches_ptrs_tensor, src_tensor,
+         block_token_indices, src_block_indices, num_tokens_per_block, dim_size_per_token_per_layer, sm_count,
+         pool_token_slots)
 
 
 def paged_gather_kv_caches(kv_caches_ptrs_tensor, dst_tensor, run_start_slots: IndexArg,

@@ -41,21 +41,41 @@ def golden():
         return json.load(f)
 
 
+class _GeneralLoaderLib:
+    """The shipped library with its three block-key entry points replaced by those of
+    tests/libkvcm_hash_general_loader.so: the same source built with KVCM_TEST_FORCE_GENERAL_LOADER=1, in which every
+    launch takes the loader form of a workgroup whose requests span 4 GiB or more."""
+    _SWAPPED = ("kvcm_hip_hash_tokens", "kvcm_hip_hash_tokens_i32", "kvcm_hip_prefix_chain")
+
+    def __init__(self):
+        import ctypes
+        from tair_kvcache_amd import _lib, build
+        if not os.path.exists(build.TEST_HOOK_LIB_PATH):
+            raise _lib.KvcmLibraryError(f"{build.TEST_HOOK_LIB_PATH} is not built; run `python -m tair_kvcache_amd.build`")
+        self._shipped = _lib.lib()
+        general = ctypes.CDLL(build.TEST_HOOK_LIB_PATH)
+        for name in self._SWAPPED:
+            fn = getattr(general, name)
+            fn.restype, fn.argtypes = _lib.SIGNATURES[name]
+            setattr(self, name, fn)
+
+    def __getattr__(self, name):  # everything else is the shipped library's
+        return getattr(self._shipped, name)
+
+
 @pytest.fixture
-def force_general_hash_loader():
-    """Switches the block-key kernel to the loader form it uses when a workgroup's requests span 4 GiB or more, through
-    the library's test hook (an exported symbol that no header declares); restores the previous setting afterwards."""
-    import ctypes
-    from tair_kvcache_amd import _lib
-    hook = _lib.lib().kvcm_test_hook_hash_force_global_loads
-    hook.restype, hook.argtypes = ctypes.c_int32, [ctypes.c_int32]
-    state = {"previous": None}
+def force_general_hash_loader(monkeypatch):
+    """switch(True) makes tair_kvcache_amd.hashing launch the block-key kernels of the general-loader build for the
+    rest of the test; switch(False) goes back to the shipped library."""
+    from tair_kvcache_amd import _torch_util, hashing
+    state = {}
 
     def switch(on):
-        previous = hook(1 if on else 0)
-        if state["previous"] is None:
-            state["previous"] = previous
+        if on:
+            if "lib" not in state:
+                state["lib"] = _GeneralLoaderLib()
+            monkeypatch.setattr(hashing, "lib", lambda: state["lib"])
+        else:
+            monkeypatch.setattr(hashing, "lib", _torch_util.lib)
 
     yield switch
-    if state["previous"] is not None:
-        hook(state["previous"])

@@ -18,6 +18,7 @@ def test_header_declares_the_expected_entry_points():
     names = declared_symbols()
     for must in ("kvcm_hip_hash_tokens", "kvcm_hip_hash_tokens_i32", "kvcm_hip_prefix_chain",
                  "kvcm_hip_sha256_first8_be", "kvcm_hip_batch_gather", "kvcm_hip_batch_scatter",
+                 "kvcm_hip_batch_gather_host_idx", "kvcm_hip_batch_scatter_host_idx",
                  "kvcm_hip_paged_gather", "kvcm_hip_paged_scatter", "kvcm_hip_gather_ex", "kvcm_hip_scatter_ex",
                  "kvcm_hip_generate_blocks_idx", "kvcm_hip_iov_crc32", "kvcm_blocks_hash_from_crcs",
                  "kvcm_hip_first_occurrence", "kvcm_hip_first_occurrence_workspace_bytes",
@@ -75,6 +76,21 @@ def test_argument_validation_needs_no_device():
     assert L.kvcm_hip_mask_to_indices_workspace_bytes(1025) == 3 * 4
     assert L.kvcm_hip_mask_to_indices(p, None, 5, p, 1 << 20, p, None, None) == _lib.ERR_INVALID_ARG  # no count
     assert L.kvcm_hip_mask_to_indices(p, None, (1 << 30) + 1, p, 1 << 20, p, p, None) == _lib.ERR_TOO_LARGE
+    # host index lists: the walk over the lists refuses a wild index before any HIP call
+    T = 16
+    tok = (ctypes.c_int32 * (2 * T))(*range(2 * T))
+    sl = (ctypes.c_int32 * 2)(0, 1)
+    host_idx = L.kvcm_hip_batch_gather_host_idx
+    assert host_idx(p, 2, p, 2 * T * 64, 2, tok, sl, 2, T, 64, 2 * T - 1, 0, None) == _lib.ERR_OUT_OF_RANGE  # token slot
+    assert host_idx(p, 2, p, 2 * T * 64, 1, tok, sl, 2, T, 64, 0, 0, None) == _lib.ERR_OUT_OF_RANGE  # staging slot
+    assert host_idx(p, 2, p, 2 * T * 64, 1, tok, None, 2, T, 64, 0, 0, None) == _lib.ERR_OUT_OF_RANGE  # implied slot 1
+    sl[1] = -1
+    assert L.kvcm_hip_batch_scatter_host_idx(p, 2, p, 2 * T * 64, 0, tok, sl, 2, T, 64, 0, 0, None) == _lib.ERR_OUT_OF_RANGE
+    assert host_idx(p, 2, p, 2 * T * 64, 2, None, sl, 2, T, 64, 0, 0, None) == _lib.ERR_INVALID_ARG
+    assert host_idx(p, 2, p, 2 * T * 64, 2, tok, sl, 0, T, 64, 0, 0, None) == _lib.OK
+    wide = (ctypes.c_int32 * 1024)(*range(0, 2048, 2))  # 1024 runs in one block: more than an argument block holds
+    assert host_idx(p, 2, p, 2 * 1024 * 64, 1, wide, None, 1, 1024, 64, 0, 0, None) == _lib.ERR_TOO_LARGE
+    assert _lib.error_string(_lib.ERR_OUT_OF_RANGE) == "index out of range"
     assert _lib.error_string(_lib.ERR_INVALID_ARG) == "invalid argument"
     assert _lib.error_string(0) == "ok"
 

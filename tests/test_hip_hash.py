@@ -81,7 +81,7 @@ def test_ragged_batch_and_seed(oracle):
 @pytest.mark.parametrize("dtype", [np.int64, np.int32])
 def test_general_loader_path(oracle, force_general_hash_loader, dtype):
     """The loader form used when a workgroup's requests span 4 GiB or more (32-bit buffer offsets cannot reach),
-    forced here through its test hook, on a ragged batch whose last request ends exactly at the end of the buffer."""
+    taken here from the test-only build in which every launch uses it, on a ragged batch whose last request ends exactly at the end of the buffer."""
     force_general_hash_loader(True)
     rng = np.random.default_rng(17)
     lens = [int(x) for x in rng.integers(0, 900, size=150)] + [64]

@@ -113,13 +113,17 @@ def test_operators_reject_host_tensors_before_touching_the_device():
 
 def test_signatures_match_the_reference_operators():
     import inspect
+    def positional(sig):  # what a reference call site can reach; extras of this port are keyword-only
+        return [n for n, p in sig.parameters.items() if p.kind is not inspect.Parameter.KEYWORD_ONLY]
+
     sig = inspect.signature(bgs.batch_gather_kv_caches)
-    assert list(sig.parameters) == ["kv_caches_ptrs_tensor", "dst_tensor", "block_token_indices", "dst_block_indices",
-                                    "num_tokens_per_block", "dim_size_per_token_per_layer", "sm_count"]
+    assert positional(sig) == ["kv_caches_ptrs_tensor", "dst_tensor", "block_token_indices", "dst_block_indices",
+                               "num_tokens_per_block", "dim_size_per_token_per_layer", "sm_count"]
     assert sig.parameters["sm_count"].default == 3
+    assert sig.parameters["pool_token_slots"].default == 0
     sig = inspect.signature(bgs.batch_scatter_kv_caches)
-    assert list(sig.parameters) == ["kv_caches_ptrs_tensor", "src_tensor", "block_token_indices", "src_block_indices",
-                                    "num_tokens_per_block", "dim_size_per_token_per_layer", "sm_count"]
+    assert positional(sig) == ["kv_caches_ptrs_tensor", "src_tensor", "block_token_indices", "src_block_indices",
+                               "num_tokens_per_block", "dim_size_per_token_per_layer", "sm_count"]
     assert list(inspect.signature(gsh.gather_kv_caches).parameters) == ["kv_caches_ptrs", "total_token_in_kvcache",
                                                                          "dst_tensor", "token_indices"]
     assert list(inspect.signature(gsh.scatter_kv_caches).parameters) == ["kv_caches_ptrs", "total_token_in_kvcache",
