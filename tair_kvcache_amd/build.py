@@ -3,10 +3,12 @@
 Every source is compiled to an object of its own, the objects in parallel, then linked. build_library() also builds
 tests/libkvcm_hash_general_loader.so: the block-key entry points compiled with KVCM_TEST_FORCE_GENERAL_LOADER, so that
 the parity tests can run the loader form that a workgroup spanning 4 GiB of tokens takes without allocating 4 GiB --
-a library of its own, because the shipped one has no switch for it."""
+a library of its own, because the shipped one has no switch for it -- and the small CPython extension
+_kvcm_pylist (gcc) that packs Python index lists."""
 import os
 import subprocess
 import sys
+import sysconfig
 from concurrent.futures import ThreadPoolExecutor
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
@@ -14,8 +16,10 @@ ROOT = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libkvcm_hip.so")
 TEST_HOOK_LIB_PATH = os.path.join(ROOT, "tests", "libkvcm_hash_general_loader.so")
-SOURCES = ["kvcm_copy.hip", "kvcm_hash.hip", "kvcm_select.hip", "kvcm_file.hip"]
+SOURCES = ["kvcm_copy.hip", "kvcm_hash.hip", "kvcm_select.hip", "kvcm_file.hip", "kvcm_host.hip"]
 OBJ_DIR = os.path.join(PKG_DIR, "build")
+# CPython extension (host code, gcc): Python index lists -> packed int32 in one C loop
+PYLIST_PATH = os.path.join(PKG_DIR, "_kvcm_pylist" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
 
 
 def _hipcc():
@@ -51,6 +55,8 @@ def build_library(verbose=False):
     link = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC"]
     outs.append(_run(link + ["-o", LIB_PATH] + [j[1] for j in jobs[:len(SOURCES)]]))
     outs.append(_run(link + ["-o", TEST_HOOK_LIB_PATH, hook_obj]))
+    outs.append(_run([os.environ.get("CC", "gcc"), "-O2", "-shared", "-fPIC", "-Wall", "-Wextra",
+                      "-I" + sysconfig.get_paths()["include"], "-o", PYLIST_PATH, os.path.join(CSRC, "kvcm_pylist.c")]))
     if verbose:
         text = "\n".join(o for o in outs if o.strip())
         if text:

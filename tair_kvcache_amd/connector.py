@@ -16,7 +16,6 @@ is whatever object offers send(bytes) (TpCoordinatorClient, kv_cache_manager/py_
 import math
 import threading
 import time
-from array import array
 from concurrent.futures import ThreadPoolExecutor
 from dataclasses import dataclass
 from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
@@ -225,13 +224,8 @@ class DataTransferManager:
         if isinstance(block_token_indices, torch.Tensor):
             return block_token_indices
         if len(block_token_indices) > 0 and isinstance(block_token_indices[0], (list, tuple)):
-            flat = array("i")  # what the operator would turn a flat list into anyway, built row by row
-            try:
-                for row in block_token_indices:
-                    flat.extend(row)
-            except (TypeError, OverflowError) as e:
-                raise ValueError(f"block_token_indices must hold ints that fit 32 bits: {e}") from e
-            return flat
+            # nested, one list per block, as generate_blocks_idx returns it in the reference: packed in one C loop
+            return batch_gather_scatter_helper.pack_index_list(block_token_indices, "block_token_indices")
         return block_token_indices
 
     def _slot_buffers(self, slot_indices):

@@ -35,6 +35,8 @@
 
 #include <cstdlib>
 
+#include "kvcm_host_idx.h"
+
 namespace kvcm {
 namespace {
 
@@ -185,10 +187,6 @@ enum RunMode { kRunPerThread = 0, kRunPerWave = 1, kRunPerGroup = 2 };
 // KernargIdx: the tables travel INSIDE the kernel's argument block, run starts first, staging slots behind them -- the
 // form behind the entry points that take host index lists: nothing is uploaded, nothing has to outlive the call, and a
 // uniform read of the table is a scalar load from the argument segment like any other kernel argument.
-constexpr int kEmbedInts = 832;  // 3328 bytes of the 4 KiB a kernel's argument block may have
-struct EmbeddedIdx {
-    int32_t v[kEmbedInts];
-};
 struct PtrIdx {
     const int32_t *run_start;
     const int32_t *staging_idx;
@@ -571,41 +569,12 @@ int32_t launch_copy_host_idx(const void *const *d_ptr_table, int32_t P, void *d_
     if (!h_token_idx || !d_ptr_table || !d_staging) {
         return KVCM_ERR_INVALID_ARG;
     }
-    // r = gcd(T, every position inside a block where the slot is not its predecessor's + 1)
-    const auto gcd = [](uint32_t x, uint32_t y) {
-        while (y) {
-            const uint32_t t = x % y;
-            x = y;
-            y = t;
-        }
-        return x;
-    };
-    uint32_t r = static_cast<uint32_t>(T);
-    const int64_t pool_limit = pool_slots > 0 ? pool_slots : (int64_t{1} << 31);
-    for (int32_t b = 0; b < B; ++b) {
-        const int32_t *row = h_token_idx + static_cast<int64_t>(b) * T;
-        if (row[0] >= pool_limit) {
-            return KVCM_ERR_OUT_OF_RANGE;
-        }
-        for (int32_t j = 1; j < T; ++j) {
-            if (row[j] >= pool_limit) {
-                return KVCM_ERR_OUT_OF_RANGE;
-            }
-            // a negative slot means "skip this row": it never joins a run, so that nothing but that row is skipped
-            if (r > 1 && (row[j - 1] < 0 || row[j] != row[j - 1] + 1)) {
-                r = gcd(r, static_cast<uint32_t>(j));
-            }
-        }
-        if (h_staging_idx) {
-            const int64_t sb = h_staging_idx[b];
-            if (sb < 0 || (staging_slots > 0 && sb >= staging_slots)) {
-                return KVCM_ERR_OUT_OF_RANGE;
-            }
-        } else if (staging_slots > 0 && b >= staging_slots) {
-            return KVCM_ERR_OUT_OF_RANGE;
-        }
+    int32_t r = 0;
+    const int32_t walked = walk_host_idx(h_token_idx, h_staging_idx, B, T, pool_slots, staging_slots, &r);
+    if (walked != KVCM_OK) {
+        return walked;
     }
-    const int32_t runs = T / static_cast<int32_t>(r);
+    const int32_t runs = T / r;
     if (runs + 1 > kEmbedInts) {
         return KVCM_ERR_TOO_LARGE;  // one block's table does not fit an argument block: upload it instead
     }
@@ -613,14 +582,8 @@ int32_t launch_copy_host_idx(const void *const *d_ptr_table, int32_t P, void *d_
     EmbeddedIdx emb;
     for (int32_t b0 = 0; b0 < B; b0 += per_launch) {
         const int32_t nb = B - b0 < per_launch ? B - b0 : per_launch;
-        for (int32_t i = 0; i < nb; ++i) {
-            const int32_t *row = h_token_idx + static_cast<int64_t>(b0 + i) * T;
-            for (int32_t k = 0; k < runs; ++k) {
-                emb.v[i * runs + k] = row[k * static_cast<int32_t>(r)];
-            }
-            emb.v[nb * runs + i] = h_staging_idx ? h_staging_idx[b0 + i] : b0 + i;
-        }
-        kvcm_copy_desc d = flat_desc(d_ptr_table, P, d_staging, block_stride, nullptr, static_cast<int32_t>(r), nullptr,
+        fill_embedded(&emb, h_token_idx, h_staging_idx, b0, nb, T, r);
+        kvcm_copy_desc d = flat_desc(d_ptr_table, P, d_staging, block_stride, nullptr, r, nullptr,
                                      nb, T, row_bytes, max_workgroups);
         const int32_t rc = launch_copy(&d, scatter, stream, &emb, static_cast<uint32_t>(nb * runs));
         if (rc != KVCM_OK) {

@@ -877,27 +877,6 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
 
 extern "C" {
 
-int32_t kvcm_hip_version(void) { return 200; }  // 0.2.0: host-index gather/scatter added, test hook gone
-
-const char *kvcm_hip_error_string(int32_t code) {
-    switch (code) {
-        case KVCM_OK:
-            return "ok";
-        case KVCM_ERR_INVALID_ARG:
-            return "invalid argument";
-        case KVCM_ERR_ALIGNMENT:
-            return "misaligned address or stride";
-        case KVCM_ERR_TOO_LARGE:
-            return "size exceeds the launch geometry";
-        case KVCM_ERR_IO:
-            return "file input/output error";
-        case KVCM_ERR_OUT_OF_RANGE:
-            return "index out of range";
-        default:
-            return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown kvcm error";
-    }
-}
-
 int32_t kvcm_hip_hash_tokens(const int64_t *d_tokens, const int64_t *d_token_offsets, int32_t R, int32_t block_size,
                              int64_t seed, int64_t *d_keys, const int64_t *d_key_offsets, kvcm_stream_t stream) {
     return kvcm::launch_hash<int64_t>(d_tokens, d_token_offsets, R, block_size, seed, d_keys, d_key_offsets,
@@ -949,21 +928,6 @@ int32_t kvcm_hip_iov_crc32(const kvcm_iov_device *d_iovs, int32_t n, uint32_t *d
     hipLaunchKernelGGL(kvcm::iov_crc32_kernel, dim3((n + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
                        d_iovs, n, d_crc, cal_bytes);
     return kvcm::launch_status();
-}
-
-int32_t kvcm_blocks_hash_from_crcs(const uint32_t *crcs, int64_t n_crcs, int32_t iovs_per_block, int64_t *out_hashes) {
-    if (iovs_per_block <= 0 || n_crcs < 0 || (n_crcs > 0 && (!crcs || !out_hashes))) {
-        return KVCM_ERR_INVALID_ARG;
-    }
-    int64_t nb = 0;
-    for (int64_t off = 0; off + iovs_per_block <= n_crcs; off += iovs_per_block) {
-        uint64_t h = 0;
-        for (int32_t i = 0; i < iovs_per_block; ++i) {
-            h = kvcm::hash_step_preadded(h, static_cast<uint64_t>(crcs[off + i]) + kvcm::kGolden);
-        }
-        out_hashes[nb++] = static_cast<int64_t>(h);
-    }
-    return KVCM_OK;
 }
 
 }  // extern "C"

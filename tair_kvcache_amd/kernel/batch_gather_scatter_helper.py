@@ -22,6 +22,11 @@ import torch
 from .. import _lib
 from .._torch_util import as_device_i32, lib, ptr, require_cuda, stream_handle
 
+try:  # one C loop over a list (flat or nested); absent only when the package was not built with its build.py
+    from .._kvcm_pylist import pack_i32 as _pack_i32
+except ImportError:  # host-side convenience only: the lists then go through array('i'), three times slower
+    _pack_i32 = None
+
 IndexArg = Union[List[int], Sequence[int], torch.Tensor]
 
 # When True, `sm_count` caps the grid as in the reference; when False the device is filled.
@@ -70,9 +75,24 @@ def _prepare(kv_caches_ptrs_tensor, staging, block_token_indices, block_indices,
     return device, P, T, row_bytes, block_bytes, tidx, sidx, B
 
 
+def pack_index_list(values, name="index list"):
+    """A Python list of ints -- flat, or nested as generate_blocks_idx returns it in the reference (one list per
+    block) -- as packed int32 in host memory: bytes, or an array('i') when the C helper is not built."""
+    try:
+        if _pack_i32 is not None and isinstance(values, (list, tuple)):
+            return _pack_i32(values)
+        if isinstance(values, (list, tuple)) and len(values) > 0 and isinstance(values[0], (list, tuple)):
+            flat = array("i")
+            for row in values:
+                flat.extend(row)
+            return flat
+        return array("i", values)
+    except (TypeError, OverflowError) as e:
+        raise ValueError(f"{name} must be a list of ints that fit 32 bits, or an integer tensor: {e}") from e
+
+
 def _host_i32(values, name):
-    """(address, count, keep-alive) of `values` as int32 in host memory, or None when `values` lives on the GPU.
-    A list goes through array('i'): one C loop over the list, a third of the time of building a tensor from it."""
+    """(address, count, keep-alive) of `values` as int32 in host memory, or None when `values` lives on the GPU."""
     if isinstance(values, torch.Tensor):
         if values.is_cuda:
             return None
@@ -80,11 +100,13 @@ def _host_i32(values, name):
         if t.dtype != torch.int32 or not t.is_contiguous():
             t = t.to(torch.int32).contiguous()
         return t.data_ptr(), t.numel(), t
-    try:
-        a = values if isinstance(values, array) and values.typecode == "i" else array("i", values)
-    except (TypeError, OverflowError) as e:
-        raise ValueError(f"{name} must be a list of ints that fit 32 bits, or an integer tensor: {e}") from e
-    return a.buffer_info()[0], len(a), a
+    if isinstance(values, bytes):  # already packed by pack_index_list
+        return values, len(values) // 4, values
+    if not (isinstance(values, array) and values.typecode == "i"):
+        values = pack_index_list(values, name)
+        if isinstance(values, bytes):
+            return values, len(values) // 4, values
+    return values.buffer_info()[0], len(values), values
 
 
 def _run(host_fn, device_fn, kv_caches_ptrs_tensor, staging, block_token_indices, block_indices,

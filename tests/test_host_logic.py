@@ -332,3 +332,31 @@ def test_hashing_and_buffer_check_reject_bad_arguments_before_any_launch():
     with pytest.raises(ValueError):   # an iov without an address
         buffer_check.get_iovs_crc([(0x1000, 64), (0, 64)], device="cpu")
     assert buffer_check.get_iovs_crc([(0x1000, 1)], device="cpu") == []            # size 1 -> nothing to hash
+
+
+def test_index_lists_are_packed_in_c_flat_and_nested():
+    """pack_index_list: the C helper and the array('i') path it replaces give the same bytes; what is not an integer
+    that fits 32 bits is refused with ValueError either way."""
+    from array import array
+    import numpy as np
+    assert bgs._pack_i32 is not None, "tair_kvcache_amd/_kvcm_pylist is not built (python -m tair_kvcache_amd.build)"
+    flat = [(i * 7919) % 500000 - 3 for i in range(2048)]
+    nested = [flat[i * 16:(i + 1) * 16] for i in range(128)]
+    want = array("i", flat).tobytes()
+    for form in (flat, tuple(flat), nested, [tuple(r) for r in nested], tuple(nested)):
+        assert bgs.pack_index_list(form) == want
+    assert bgs.pack_index_list([np.int64(5), True, -2 ** 31, 2 ** 31 - 1]) == array("i", [5, 1, -2 ** 31, 2 ** 31 - 1]).tobytes()
+    assert bgs.pack_index_list([]) == b"" and bgs.pack_index_list([[], []]) == b""
+    for bad in ([1.5], [2 ** 31], [-2 ** 31 - 1], ["7"], [[1], 2], [None], [[1.0]]):
+        with pytest.raises(ValueError):
+            bgs.pack_index_list(bad)
+    # the same without the C helper
+    helper, bgs._pack_i32 = bgs._pack_i32, None
+    try:
+        assert bytes(bgs.pack_index_list(flat)) == want and bgs.pack_index_list(nested).tobytes() == want
+        assert bgs.pack_index_list(range(5)).tolist() == [0, 1, 2, 3, 4]
+        for bad in ([1.5], [2 ** 31], ["7"], [[1], 2]):
+            with pytest.raises(ValueError):
+                bgs.pack_index_list(bad)
+    finally:
+        bgs._pack_i32 = helper
