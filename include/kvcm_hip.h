@@ -297,6 +297,10 @@ typedef struct kvcm_iov_device {
  * Replaces: GetIovsCrcDevice  kv_cache_manager/client/src/internal/sdk/sdk_buffer_check_util.cu:21-44
  * (the caller picks cal_bytes = min(KVCM_CHECK_IOV_BYTE_SIZE, iovs[0].size / 2) and skips the launch
  * when it is 0, as sdk_buffer_check_util.cu:50-55 does).
+ * Contract for an iov with base == NULL or size < cal_bytes (the reference reads out of bounds there, so there is no
+ * behaviour to match): the kernel reads nothing of it and writes d_crc[i] = 0. Because 0 is also a valid CRC, a
+ * caller that cannot rule such iovs out validates them on the host before the launch: kvcm::IovCheckBytes
+ * (kvcm_hip.hpp) returns 0 = "check nothing" for the whole call, the Python layer raises ValueError.
  */
 int32_t kvcm_hip_iov_crc32(const kvcm_iov_device *d_iovs, int32_t n, uint32_t *d_crc,
                            size_t cal_bytes, kvcm_stream_t stream);

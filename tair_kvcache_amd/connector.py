@@ -28,6 +28,40 @@ from .kernel import batch_gather_scatter_helper
 from .kernel.gather_scatter_helper import CopyBufferAllocator
 
 
+_blocks_idx_error_flags: Dict[Any, torch.Tensor] = {}
+_blocks_idx_error_lock = threading.Lock()
+
+
+def _default_error_flag(device: torch.device) -> torch.Tensor:
+    """The int32 flag that generate_blocks_idx raises for tensor arguments when the caller passes none: one per
+    device, created on first use, read and cleared by blocks_idx_error()."""
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    flag = _blocks_idx_error_flags.get(key)
+    if flag is None:
+        with _blocks_idx_error_lock:
+            flag = _blocks_idx_error_flags.get(key)
+            if flag is None:
+                flag = torch.zeros(1, dtype=torch.int32, device=device)
+                _blocks_idx_error_flags[key] = flag
+    return flag
+
+
+def blocks_idx_error(device="cuda", clear: bool = True) -> bool:
+    """True when a generate_blocks_idx call with tensor arguments (and no error_flag of its own) on `device` has met a
+    manager block that reaches beyond local_block_ids since the last call of this function. Reads the flag back, so
+    it waits for the device: call it at a point where the caller waits anyway (DataTransferManager.save_task does,
+    after the event it waits for and before the staged blocks are handed to the transfer client)."""
+    device = torch.device(device)
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    flag = _blocks_idx_error_flags.get(key)
+    if flag is None:
+        return False
+    raised = bool(flag.item())
+    if raised and clear:
+        flag.zero_()
+    return raised
+
+
 def generate_blocks_idx(manager_block_idxes: Sequence[int], local_block_ids: Sequence[int],
                         manager_block_size: int, local_block_size: int, device="cuda",
                         error_flag: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -38,8 +72,10 @@ def generate_blocks_idx(manager_block_idxes: Sequence[int], local_block_ids: Seq
 
     A manager block that reaches beyond local_block_ids: with Python sequences this raises AssertionError before
     anything is launched, as the reference's assert does. With tensor arguments nothing is read back (no
-    synchronisation): the kernel writes -1 for such entries, which the gather/scatter kernels skip, and raises
-    `error_flag` (an int32 device tensor of one element, if given) to 1."""
+    synchronisation): the kernel writes -1 for such entries, which the gather/scatter kernels skip, and raises an
+    int32 flag on the device to 1 -- `error_flag` if the caller passes one, otherwise a flag the module keeps per
+    device, which blocks_idx_error() reads and clears. The error is never dropped: DataTransferManager.save_task looks
+    at that flag before it lets the transfer client save what was gathered."""
     T_mgr, T_eng = int(manager_block_size), int(local_block_size)
     B = len(manager_block_idxes)
     out = torch.empty((B, T_mgr), dtype=torch.int32, device=device)
@@ -51,6 +87,8 @@ def generate_blocks_idx(manager_block_idxes: Sequence[int], local_block_ids: Seq
             raise AssertionError("manager block reaches beyond local_block_ids")
     if error_flag is not None and (not error_flag.is_cuda or error_flag.dtype != torch.int32 or error_flag.numel() < 1):
         raise ValueError("error_flag must be an int32 tensor on the GPU")
+    if error_flag is None and isinstance(manager_block_idxes, torch.Tensor):
+        error_flag = _default_error_flag(out.device)
     m = as_device_i32(manager_block_idxes, out.device, "manager_block_idxes")
     l = as_device_i32(local_block_ids, out.device, "local_block_ids")
     rc = lib().kvcm_hip_generate_blocks_idx(ptr(m), B, ptr(l), l.numel(), T_mgr, T_eng, ptr(out), ptr(error_flag),
@@ -321,7 +359,13 @@ class DataTransferManager:
                 done = torch.cuda.Event()
                 done.record(self._save_stream)
             done.synchronize()
-            result = self._transfer_client.SaveKvCaches(remote_uris, self._slot_buffers(slots))
+            if isinstance(block_token_indices, torch.Tensor) and block_token_indices.is_cuda and \
+                    blocks_idx_error(block_token_indices.device):
+                # indices built on the device named a block beyond the request's block list: those rows were skipped
+                # by the gather, so the staged bytes are not the request's KV cache and must not be saved
+                result = (self._cm.ClientErrorCode.ER_INVALID_PARAMS, [])
+            else:
+                result = self._transfer_client.SaveKvCaches(remote_uris, self._slot_buffers(slots))
         finally:
             if slots is not None:
                 self._copy_buffer_allocator.free_buffer(slots)

@@ -251,7 +251,10 @@ __device__ __forceinline__ void copy_span_body(const CopyArgs &a, const void *co
         V v[kCPT];
         unsigned char *pp[kCPT];
         unsigned char *sp[kCPT];
-        uint32_t tr_word = 0;             // a 4-byte trailer in flight, and where it goes
+        // a 4-byte trailer in flight, and where it goes: one per thread, which is enough because a thread owns one
+        // chunk -- with several chunks per thread on the non-uniform path a thread could own the first chunk of two tiles
+        static_assert(kCPT == 1, "the 4-byte trailer path keeps one trailer per thread");
+        uint32_t tr_word = 0;
         unsigned char *tr_dst = nullptr;
 #pragma unroll
         for (int u = 0; u < kCPT; ++u) {

@@ -342,6 +342,8 @@ template <typename Loader, typename TokT, int KS, int G>
 __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t (*s_tile)[kReqs][kTT + kPad],
                                            int64_t lw, int64_t ntiles, uint32_t lane, const KeyDrain &kd) {
     static_assert(kRing == 2 && kLoaders >= 3, "two ring slots: prefetched from, written to");
+    // the burst drain splits a closed group between the kLoaders - 1 loaders whose tile is not due, as halves
+    static_assert(KS != kKeysBurst || kLoaders == 3, "drain_half deals a group out to exactly two loaders");
     static_assert((G & (G - 1)) == 0 && (KS != kKeysSpread || G == kKeyGroupTiles), "groups of 2^n tiles; spread: 16");
     Loader ld;
     ld.setup(ctx, lane);
@@ -736,7 +738,8 @@ __global__ __launch_bounds__(256) void iov_crc32_kernel(const kvcm_iov_device *_
     const size_t size = iovs[i].size;
     if (!p || size < cal_bytes) {
         // cal_bytes comes from the first iov only: an iov without an address, or shorter than that, is not read at
-        // all and gets the value 0 (the reference reads out of bounds here)
+        // all and gets the value 0 (the reference reads out of bounds here). 0 is also a possible CRC, so callers
+        // that cannot rule such iovs out check them on the host first, as the C++ and Python layers above do.
         out[i] = 0;
         return;
     }

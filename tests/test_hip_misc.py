@@ -448,3 +448,38 @@ def test_transfer_manager_with_staging_in_hbm(oracle):
     assert alloc._inuse_count == 0
     mgr.shutdown()
     mgr2.shutdown()
+
+
+def test_device_built_indices_that_leave_the_block_list_are_not_saved():
+    """generate_blocks_idx with tensor arguments never reads back; a manager block beyond local_block_ids (the reference
+    asserts, v1_connector.py:316) raises the module's per-device flag instead, and save_task, which waits for its gather
+    anyway, looks at the flag before it hands the staged blocks to the transfer client."""
+    from tair_kvcache_amd import connector
+    from tair_kvcache_amd.client_types import ClientErrorCode
+    from tair_kvcache_amd.kernel.gather_scatter_helper import CopyBufferAllocator
+    L, nblk, T, H, hd = 2, 16, 16, 2, 32
+    kv = {f"layer{l}": torch.ones(2, nblk, T, H, hd, dtype=torch.bfloat16, device="cuda") for l in range(L)}
+    info = connector.register_kv_caches(kv, T, T)
+    # pinned host staging: the fake client reads the slots with the CPU
+    alloc = CopyBufferAllocator(torch.device("cpu"), torch.bfloat16, list(info.per_manager_block_shape), 8)
+    client = FakeTransferClient()
+    mgr = connector.DataTransferManager(info, T, alloc, client, max_workers=2)
+    connector.blocks_idx_error("cuda")  # whatever an earlier test left behind
+    assert connector.blocks_idx_error("cuda") is False
+    local = torch.tensor([3, 5, 7], dtype=torch.int32, device="cuda")
+    good = connector.generate_blocks_idx(torch.tensor([0, 2], dtype=torch.int32, device="cuda"), local, T, T)
+    assert connector.blocks_idx_error("cuda") is False
+    bad = connector.generate_blocks_idx(torch.tensor([1, 3], dtype=torch.int32, device="cuda"), local, T, T)
+    sync()
+    assert host(bad, np.int32)[1].tolist() == [-1] * T and host(good, np.int32)[1, 0] == 7 * T
+    for idx, want in ((bad, ClientErrorCode.ER_INVALID_PARAMS), (good, ClientErrorCode.ER_OK)):
+        done, out = threading.Event(), []
+        multi = connector.MultiResult(1, lambda r: (out.append(r), done.set()))
+        uris = [f"file:///kv/err?blkid={i}&size={info.per_manager_block_byte_size}" for i in range(2)]
+        mgr.submit_task(mgr.save_task, multi, 0, uris, idx)
+        assert done.wait(60)
+        assert out[0] == [[want] * 2]
+        assert alloc._inuse_count == 0
+        assert (want == ClientErrorCode.ER_OK) == all(u in client.store for u in uris)
+    assert connector.blocks_idx_error("cuda") is False  # read and cleared by the task that met it
+    mgr.shutdown()
