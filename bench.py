@@ -182,6 +182,10 @@ def other_configs(torch, np, device, reps=5):
         torch.cuda.synchronize()
         torch.cuda.empty_cache()
 
+    def sample_blocks(B, n=64):  # first, last and a seeded sample: what every configuration's result is checked on
+        picks = np.random.default_rng(6).choice(B, size=min(n, B), replace=False).tolist()
+        return sorted(set(picks + [0, B - 1]))
+
     def tokens_uniform(R, L, vocab, seed=0):
         return torch.from_numpy(np.random.default_rng(seed).integers(0, vocab, size=(R, L), dtype=np.int64)).to(device)
 
@@ -209,7 +213,7 @@ def other_configs(torch, np, device, reps=5):
         ms_g = gpu_ms(torch, lambda: launch(L.kvcm_hip_paged_gather, d_save), n)
         ms_s = gpu_ms(torch, lambda: launch(L.kvcm_hip_paged_scatter, d_load), n)
         ok = True
-        for b in (0, B // 2, B - 1):
+        for b in sample_blocks(B):
             s0, l0 = int(save_b[b]) * Tb, int(load_b[b]) * Tb
             ok &= bool(torch.equal(staging[b], pool[:, s0:s0 + Tb])) and bool(torch.equal(staging[b], pool[:, l0:l0 + Tb]))
         _, hf = hash_figures(torch, hashing, tok, hash_block, 10)
@@ -226,6 +230,14 @@ def other_configs(torch, np, device, reps=5):
     paged("C1", "Qwen2-0.5B-like: 24 layers x K/V, 2 KV heads x 64, bf16, 16-token blocks, pool of 1024 blocks, 128 "
           "blocks moved (2 x 24 MiB per launch: launch-latency bound); 4 requests x 512 tokens hashed",
           48, 128, 16, 1024, perm[:128], perm[128:256], torch.from_numpy(tok).to(device), 16)
+
+    # C2 under tensor parallelism 8: one rank's share of the Llama-3-8B cache, 1 KV head = 256-byte rows, 4 KiB tiles
+    perm = np.random.default_rng(2).permutation(32768).astype(np.int32)
+    tok = np.random.default_rng(0).integers(0, VOCAB, size=(REQUESTS, TOKENS_PER_REQ), dtype=np.int64)
+    paged("C2_tp8", "Llama-3-8B layout as one rank of TP8 sees it: 32 layers x K/V, 1 KV head x 128, bf16 (256-byte rows, "
+          "4 KiB tiles), 16-token blocks, pool of 32768 blocks; 12416 blocks saved and loaded (2 x 3.03 GiB per launch); "
+          "the keys are the request's, computed once, not per rank", 64, 128, 16, 32768, perm[:12416], perm[12416:24832],
+          torch.from_numpy(tok).to(device), 16)
 
     # C3: 72B-class, 80 layers x K/V, 8 x 128 bf16, 64-token blocks, 8192-block pool; the 25 % missed blocks of
     # 32 requests x 16384 tokens (2048 blocks, 40 GiB staged)
@@ -268,7 +280,7 @@ def other_configs(torch, np, device, reps=5):
     ms_s = gpu_ms(torch, lambda: launch(_lib.lib().kvcm_hip_scatter_ex), reps)  # a full permutation: writes every row back
     st = staging.view(nblk4, L4, rec)
     ok = True
-    for b in (0, nblk4 // 2, nblk4 - 1):
+    for b in sample_blocks(nblk4):  # payload and the 4 scale bytes behind every tile, both directions (a full permutation)
         s0 = int(blocks[b]) * T4
         ok &= bool(torch.equal(st[b, :, :T4 * row4], pool[:, s0:s0 + T4].reshape(L4, T4 * row4)))
         ok &= bool(torch.equal(st[b, :, T4 * row4:].contiguous().view(torch.float32).reshape(-1), scales[:, int(blocks[b])]))
@@ -296,7 +308,7 @@ def other_configs(torch, np, device, reps=5):
     ms_g = gpu_ms(torch, lambda: bgs.batch_gather_kv_caches(table, staging, idx_g, slots, 16, D5), reps)
     ms_s = gpu_ms(torch, lambda: bgs.batch_scatter_kv_caches(table, staging, idx_s, slots, 16, D5), reps)
     ok = True
-    for b in (0, B5 // 2, B5 - 1):
+    for b in sample_blocks(B5):
         gi, si = idx_g[b * 16:(b + 1) * 16].long(), idx_s[b * 16:(b + 1) * 16].long()
         ok &= bool(torch.equal(staging[b], pool[:, gi])) and bool(torch.equal(staging[b], pool[:, si]))
     tok5, _, _ = zipf_prefix_tokens(np)
@@ -548,7 +560,7 @@ def main():
     verified = None
     if not args.no_verify:
         # staged bytes of a sample of blocks against the pool rows they came from, and loaded rows against staging
-        sample = np.random.default_rng(3).choice(unique, size=16, replace=False)
+        sample = np.random.default_rng(3).choice(unique, size=64, replace=False)
         ok = True
         for b in sample:
             src = int(inp["save_blocks"][b]) * T
@@ -656,6 +668,27 @@ def main():
     reference_signature["through_DataTransferManager"] = manager_figures(
         torch, np, inp, args.pool_blocks, task_bytes, n_tasks, device)
 
+    # ---- the per-token-index form of the same workload: 16 x 12 416 unrelated token slots, every row (2 KiB) from
+    # a place of its own -- what page size 1 makes of this layout, and what the reference's index format always is
+    perm_slots = np.random.default_rng(7).permutation(args.pool_blocks * T).astype(np.int32)
+    tg_save = torch.from_numpy(perm_slots[:unique * T]).to(device)
+    tg_load = torch.from_numpy(perm_slots[unique * T:2 * unique * T]).to(device)
+    ms_tg_g = gpu_ms(torch, lambda: bgs.batch_gather_kv_caches(inp["ptr_table"], staging, tg_save, d_slots, T, D), 5)
+    ms_tg_s = gpu_ms(torch, lambda: bgs.batch_scatter_kv_caches(inp["ptr_table"], staging, tg_load, d_slots, T, D), 5)
+    tg_ok = None
+    if not args.no_verify:
+        tg_ok = True
+        for b in np.random.default_rng(10).choice(unique, size=64, replace=False):
+            gi, si = tg_save[b * T:(b + 1) * T].long(), tg_load[b * T:(b + 1) * T].long()
+            tg_ok &= bool(torch.equal(staging[b], inp["pool"][:, gi])) and bool(torch.equal(staging[b], inp["pool"][:, si]))
+        if not tg_ok:
+            raise SystemExit("bench.py: token-granular copy moved wrong bytes; refusing to report a number")
+    token_granular = {"workload": f"{unique * T} unrelated token slots of the same pool <-> the same {unique} staging "
+                                  "blocks (device-resident int32 index, one entry per token, 2 KiB rows)",
+                      "algorithmic_bytes_per_launch": copy_bytes + 4 * unique * T, "save": copy_figures(ms_tg_g, copy_bytes),
+                      "load": copy_figures(ms_tg_s, copy_bytes), "sample_verified": tg_ok}
+    del tg_save, tg_load
+
     # ---- the copy kernel on ONE contiguous buffer of the same size (one array, identity block table): what this chip
     # gives a read+write stream, the ceiling the random-block figures are to be read against
     flat_src = inp["pool"].view(torch.int16).reshape(-1)[:unique * P * T * D].view(1, unique * P * T, D)
@@ -679,12 +712,50 @@ def main():
                                                        key_offsets=sat_koff), 10, warm=2)
     sat_keys_per_s = sat_keys.numel() / (ms_sat * 1e-3)
     sat_alg_bytes = sat_R * TOKENS_PER_REQ * 8 + (sat_R + 1) * 8 * 2 + sat_keys.numel() * 8
+    kpr = TOKENS_PER_REQ // T  # keys per request
+
+    def check_key_sample(tokens, keys, rows, what):
+        """Keys of a seeded sample of requests of a big launch against the oracle (outside every timed region)."""
+        if args.no_verify:
+            return None
+        from oracle import oracle as O
+        pick = np.sort(np.random.default_rng(8).choice(tokens.shape[0], size=rows, replace=False))
+        d_pick = torch.from_numpy(pick).to(device)
+        want, _ = O.hash_tokens(tokens[d_pick].cpu().numpy().astype(np.int64), T, threads=min(os.cpu_count() or 1, 16))
+        got = keys.view(-1, kpr)[d_pick].cpu().numpy().reshape(-1)
+        if not bool((got == want).all()):
+            raise SystemExit(f"bench.py: {what}: keys differ from the oracle; refusing to report a number")
+        return True
+
+    sat_verified = check_key_sample(sat_tokens, sat_keys, 256, "saturated int64 launch")
+    # the same launch on 4-byte token IDs, the width engines hold them in (16 384 x 4096 x 4 B = 256 MiB of tokens)
+    sat_tokens32 = sat_tokens.to(torch.int32)
+    sat_keys.fill_(0)
+    ms_sat32 = gpu_ms(torch, lambda: hashing.hash_tokens(sat_tokens32, T, token_offsets=sat_toff, keys=sat_keys,
+                                                         key_offsets=sat_koff), 10, warm=2)
+    ms_sat32_cold = cold_ms(torch, lambda: hashing.hash_tokens(sat_tokens32, T, token_offsets=sat_toff, keys=sat_keys,
+                                                               key_offsets=sat_koff), device)
+    sat32_verified = check_key_sample(sat_tokens32, sat_keys, 256, "saturated int32 launch")
+    sat32_alg_bytes = sat_R * TOKENS_PER_REQ * 4 + (sat_R + 1) * 8 * 2 + sat_keys.numel() * 8
+    roof_hash32 = {"bound": "hbm", "achieved": round(sat32_alg_bytes / (ms_sat32 * 1e-3) / 1e9, 1),
+                   "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                   "frac": round(sat32_alg_bytes / (ms_sat32 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                   "kernel": "hash_tokens_kernel<int, 8, 16>", "ms_per_launch": round(ms_sat32, 4),
+                   "ms_per_launch_cold": round(ms_sat32_cold, 4),
+                   "frac_cold": round(sat32_alg_bytes / (ms_sat32_cold * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                   "algorithmic_bytes_per_launch": sat32_alg_bytes,
+                   "keys_per_s": round(sat_keys.numel() / (ms_sat32 * 1e-3)), "verified_against_oracle": sat32_verified,
+                   "note": "ms_per_launch repeats the launch on the same 256 MiB of tokens (the loads are non-temporal, "
+                           "so they do not stay in the 256 MiB memory-side cache); ms_per_launch_cold follows a pass "
+                           "over 2 GiB of other memory"}
+    del sat_tokens32
     # four batches of the configuration in one launch (256 chains): the smallest launch that is past 1e9 keys/s, since
     # one batch alone is bound by the latency of its 4096 dependent steps
     few_R = 4 * REQUESTS
     few_keys = few_R * (TOKENS_PER_REQ // T)
     ms_few = gpu_ms(torch, lambda: hashing.hash_tokens(sat_tokens[:few_R], T, token_offsets=sat_toff[:few_R + 1],
                                                        keys=sat_keys[:few_keys], key_offsets=sat_koff[:few_R + 1]), 10)
+    check_key_sample(sat_tokens[:few_R], sat_keys[:few_keys], few_R, "four batches in one launch")
     # the one batch of the configuration launched back to back: the step's own pair of events also times the
     # hand-over from the 8 ms load kernel before it
     ms_hash_b2b = gpu_ms(torch, hash_once, 20)
@@ -702,12 +773,23 @@ def main():
             raise SystemExit(f"bench.py: kvcm_hip_prefix_chain failed with code {rc}")
 
     ms_chain = gpu_ms(torch, chain_once, 5, warm=2)
+    chain_verified = None
+    if not args.no_verify:
+        from oracle import oracle as O
+        pick = np.sort(np.random.default_rng(9).choice(sat_R, size=256, replace=False))
+        d_pick = torch.from_numpy(pick).to(device)
+        digests = sat_tokens[d_pick].cpu().numpy()
+        want, _ = O.hash_tokens(digests, 1, threads=min(os.cpu_count() or 1, 16))  # block size 1 = the prefix chain
+        chain_verified = bool((chain_keys.view(sat_R, TOKENS_PER_REQ)[d_pick].cpu().numpy().reshape(-1) == want).all())
+        if not chain_verified:
+            raise SystemExit("bench.py: prefix chain: keys differ from the oracle; refusing to report a number")
     chain_bytes = 2 * sat_R * TOKENS_PER_REQ * 8 + (sat_R + 1) * 8
     prefix_chain = {"chains": sat_R, "digests_per_chain": TOKENS_PER_REQ, "ms_per_launch": round(ms_chain, 4),
                     "keys_per_s": round(chain_keys.numel() / (ms_chain * 1e-3)),
                     "algorithmic_bytes_per_launch": chain_bytes,
                     "GBps": round(chain_bytes / (ms_chain * 1e-3) / 1e9, 1),
-                    "frac_of_hbm_peak": round(chain_bytes / (ms_chain * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+                    "frac_of_hbm_peak": round(chain_bytes / (ms_chain * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                    "verified_against_oracle": chain_verified}
     del sat_tokens, chain_keys
 
     digest = kernel_sources_digest()
@@ -739,7 +821,7 @@ def main():
                  "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                  "frac": round(sat_alg_bytes / (ms_sat * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": sat_traffic,
                  "kernel": "hash_tokens_kernel<long, 8, 16>", "ms_per_launch": round(ms_sat, 4),
-                 "algorithmic_bytes_per_launch": sat_alg_bytes}
+                 "algorithmic_bytes_per_launch": sat_alg_bytes, "verified_against_oracle": sat_verified}
     if sat_why:
         roof_hash["traffic_null_because"] = sat_why
 
@@ -758,6 +840,7 @@ def main():
         "load_GBps": roof_s["achieved"], "load_frac_of_hbm_peak": roof_s["frac"], "load_ms": round(ms_scatter, 4),
         "per_step": per_step,
         "contiguous_copy_same_kernel": contiguous,
+        "token_granular_index": token_granular,
         "keys_per_s": round(d_keys.numel() / (ms_hash * 1e-3)), "hash_ms": round(ms_hash, 4), "hash_chains": REQUESTS,
         "hash_ms_back_to_back": round(ms_hash_b2b, 4),
         "keys_per_s_back_to_back": round(d_keys.numel() / (ms_hash_b2b * 1e-3)),
@@ -776,6 +859,7 @@ def main():
         "verified_against_oracle": verified,
         "roofline": dominant,
         "roofline_hash_saturated": roof_hash,
+        "roofline_hash_saturated_i32": roof_hash32,
         "prefix_chain_saturated": prefix_chain,
         "roofline_save": roof_g, "roofline_load": roof_s,
         "reference_signature": reference_signature,
