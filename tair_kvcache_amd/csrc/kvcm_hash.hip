@@ -29,6 +29,15 @@ namespace {
 #ifndef KVCM_HASH_LOADERS
 #define KVCM_HASH_LOADERS 3
 #endif
+#ifndef KVCM_HASH_RAW_AHEAD
+#define KVCM_HASH_RAW_AHEAD 1
+#endif
+#ifndef KVCM_HASH_BURST_ISSUE_WHOLE
+#define KVCM_HASH_BURST_ISSUE_WHOLE 1
+#endif
+#ifndef KVCM_HASH_DRAIN_POLICY
+#define KVCM_HASH_DRAIN_POLICY 0
+#endif
 #ifndef KVCM_HASH_TILE_TOKENS
 #define KVCM_HASH_TILE_TOKENS 64
 #endif
@@ -43,12 +52,17 @@ constexpr int kTT = KVCM_HASH_TILE_TOKENS;    // tokens per request per tile
 constexpr int kRing = 2;                      // LDS tiles in the ring: prefetched from, written to (the tile that is
                                               // computed on already sits in the chain wave's registers)
 constexpr int kPad = 2;                       // keeps rows 16-byte aligned (b128 reads) and spreads banks
-constexpr int kPerLane = kReqs * kTT / 64;  // tile elements per loader lane
+// Raw tiles (4-byte tokens, many requests in flight): a ring slot holds [64 requests x 128 RAW int32 tokens] -- the same
+// bytes as 64 pre-added 64-bit terms -- so that a request's share of a tile is 512 contiguous bytes of the token stream
+// instead of 256 (the memory system serves 256-byte pieces at little more than half the rate of 512-byte ones), and the
+// chain wave sign-extends and adds the constant itself, one instruction per step beside the chain.
+constexpr int tile_tokens(bool raw) { return raw ? 2 * kTT : kTT; }
+constexpr int kRowVecs = kTT / 2;  // 16-byte pieces of one request's row of a tile, either format
 // Staged keys (many requests in flight; block sizes 1, 8, 16, 32, 64 and 128): the keys of a GROUP of tiles collect in LDS
 // and leave as whole rows of 512 bytes per request, see hash_tokens_kernel. A group is as many tiles as yield 64 keys per
 // request: key_group_tiles(block size), i.e. one tile at block size 1, sixteen at block size 16, 128 at block size 128.
 constexpr int kKeysPerGroup = 64;
-constexpr int key_group_tiles(int bs) { return bs >= 1 && bs <= 2 * kTT ? kKeysPerGroup * bs / kTT : 16; }
+constexpr int key_group_tiles(int bs, int tok = kTT) { return bs >= 1 && bs <= 2 * kTT ? kKeysPerGroup * bs / tok : 16; }
 constexpr int kKeyGroupTiles = key_group_tiles(16);  // the spread form exists for block size 16 only
 static_assert(key_group_tiles(1) == 1 && key_group_tiles(16) == 16 && key_group_tiles(128) == 128, "64 keys per group");
 constexpr int kKeyPad = 2;
@@ -129,10 +143,11 @@ struct LoaderCtx {
 // workgroup's first token to the end of the batch: the hardware returns zeros past the end instead of faulting, so
 // the loads need no clamp, and a load costs two instructions (offset add + buffer_load_dwordx4). Positions past a
 // request's own last hashed token read a neighbour's tokens; the chain wave never consumes those entries.
-template <typename TokT>
+template <typename TokT, bool RAW = false>
 struct BufferLoader {
+    static_assert(!RAW || sizeof(TokT) == 4, "raw tiles hold 4-byte tokens");
     static constexpr int kEPL = 16 / sizeof(TokT);  // tokens per load
-    static constexpr int kLPR = kTT / kEPL;         // lanes per request row
+    static constexpr int kLPR = tile_tokens(RAW) / kEPL;  // lanes per request row
     static constexpr int kRPW = 64 / kLPR;          // request rows per load instruction
     static constexpr int kNL = kReqs / kRPW;        // loads per lane per tile
     __amdgpu_buffer_rsrc_t rsrc;
@@ -176,8 +191,12 @@ struct BufferLoader {
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0); lgkmcnt and expcnt left at their maxima
 #pragma unroll
         for (int j = 0; j < kNL; ++j) {
-            ulonglong2 *dst = reinterpret_cast<ulonglong2 *>(&tile[j * kRPW + sub][piece * kEPL]);
             const u32x4 v = regs[j];
+            if (RAW) {
+                reinterpret_cast<u32x4 *>(&tile[j * kRPW + sub][0])[piece] = v;  // as it came: the chain wave converts
+                continue;
+            }
+            ulonglong2 *dst = reinterpret_cast<ulonglong2 *>(&tile[j * kRPW + sub][piece * kEPL]);
             if (sizeof(TokT) == 8) {
                 dst[0] = make_ulonglong2(((static_cast<uint64_t>(v.y) << 32) | v.x) + kGolden,
                                          ((static_cast<uint64_t>(v.w) << 32) | v.z) + kGolden);
@@ -191,8 +210,10 @@ struct BufferLoader {
 
 // Loader, general form: one element per load through global addresses, positions clamped to the last token of
 // the batch. Used when the workgroup's requests span 4 GiB or more, which a 32-bit buffer offset cannot address.
-template <typename TokT>
+template <typename TokT, bool RAW = false>
 struct GlobalLoader {
+    static constexpr int kTok = tile_tokens(RAW);
+    static constexpr int kPerLane = kReqs * kTok / 64;  // tile elements per loader lane
     LoaderCtx<TokT> c;
     TokT regs[kPerLane];
     uint32_t lane;
@@ -210,7 +231,7 @@ struct GlobalLoader {
 #pragma unroll
         for (int j = HALF * (kPerLane / 2); j < (HALF + 1) * (kPerLane / 2); ++j) {
             const uint32_t e = lane + 64u * j;
-            const int64_t pos = c.s_start[e / kTT] + t0 + (e % kTT);
+            const int64_t pos = c.s_start[e / kTok] + t0 + (e % kTok);
             regs[j] = c.tokens[pos < c.last_token ? pos : c.last_token];
         }
     }
@@ -218,7 +239,11 @@ struct GlobalLoader {
 #pragma unroll
         for (int j = 0; j < kPerLane; ++j) {
             const uint32_t e = lane + 64u * j;
-            tile[e / kTT][e % kTT] = static_cast<uint64_t>(static_cast<int64_t>(regs[j])) + kGolden;
+            if (RAW) {
+                reinterpret_cast<uint32_t *>(&tile[e / kTok][0])[e % kTok] = static_cast<uint32_t>(regs[j]);
+            } else {
+                tile[e / kTok][e % kTok] = static_cast<uint64_t>(static_cast<int64_t>(regs[j])) + kGolden;
+            }
         }
     }
 };
@@ -288,7 +313,17 @@ __device__ __forceinline__ void drain_half(const KeyDrain &kd, int32_t group, in
                 // written through at system scope: 97-99 us for 16 384 x 4096 tokens where the same stores take
                 // 101-105 us non-temporal, 104 plain, 100-101 with sc1 alone (65 536 x 4096: 385-388 against 399-403 us)
                 int64_t *dst = kd.keys + first[i] + static_cast<int64_t>(group) * kKeysPerGroup + piece[i] * 2;
+#if KVCM_HASH_DRAIN_POLICY == 0
                 asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" : : "v"(dst), "v"(v[i]) : "memory");
+#elif KVCM_HASH_DRAIN_POLICY == 1
+                asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(dst), "v"(v[i]) : "memory");
+#elif KVCM_HASH_DRAIN_POLICY == 2
+                asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst), "v"(v[i]) : "memory");
+#elif KVCM_HASH_DRAIN_POLICY == 3
+                asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(dst), "v"(v[i]) : "memory");
+#else
+                asm volatile("global_store_dwordx4 %0, %1, off" : : "v"(dst), "v"(v[i]) : "memory");
+#endif
             }
         }
     }
@@ -338,7 +373,7 @@ __device__ __forceinline__ void drain_tail(const KeyDrain &kd, int32_t group, in
     }
 }
 
-template <typename Loader, typename TokT, int KS, int G>
+template <typename Loader, typename TokT, int KS, int G, int TOK>
 __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t (*s_tile)[kReqs][kTT + kPad],
                                            int64_t lw, int64_t ntiles, uint32_t lane, const KeyDrain &kd) {
     static_assert(kRing == 2 && kLoaders >= 3, "two ring slots: prefetched from, written to");
@@ -351,14 +386,14 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
     // request of 2^37 tokens does not fit the memory of the device
     const int32_t nt = static_cast<int32_t>(ntiles), me = static_cast<int32_t>(lw);
     if (me < nt) {
-        ld.issue(static_cast<int64_t>(me) * kTT);
+        ld.issue(static_cast<int64_t>(me) * TOK);
     }
     if (me < 2 && me < nt) {
         ld.store(s_tile[me]);
     }
     lds_barrier();
     if (me < 2 && me + kLoaders < nt) {
-        ld.issue(static_cast<int64_t>(me + kLoaders) * kTT);
+        ld.issue(static_cast<int64_t>(me + kLoaders) * TOK);
     }
     // tile 2 goes where tile 0 lies: not before the chain wave has pulled tile 0 into its registers
     lds_barrier();
@@ -387,17 +422,17 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
         // instructions sits in the CU's memory pipeline in front of the chain wave's key stores
         // (which of the two forms runs is a compile-time matter: with both in one loop body the compiler waits for
         // all outstanding loads where the paths meet, and a kernel that does so takes 80 us for a batch instead of 58)
-        if (KS == kKeysSpread) {
+        if (KS == kKeysSpread || (KS == kKeysBurst && KVCM_HASH_BURST_ISSUE_WHOLE && sizeof(TokT) == 8)) {
             // no key stores of the chain wave to keep out of the way of: 2 to 5 % faster from 4096 requests than in halves
             if (mine && nxt + kLoaders < nt) {
-                ld.issue(static_cast<int64_t>(nxt + kLoaders) * kTT);
+                ld.issue(static_cast<int64_t>(nxt + kLoaders) * TOK);
             }
         } else {
             if (mine && nxt + kLoaders < nt) {
-                ld.template issue_half<0>(static_cast<int64_t>(nxt + kLoaders) * kTT);
+                ld.template issue_half<0>(static_cast<int64_t>(nxt + kLoaders) * TOK);
             }
             if (was_mine && nxt - 1 + kLoaders < nt) {
-                ld.template issue_half<1>(static_cast<int64_t>(nxt - 1 + kLoaders) * kTT);
+                ld.template issue_half<1>(static_cast<int64_t>(nxt - 1 + kLoaders) * TOK);
             }
         }
         was_mine = mine;
@@ -428,21 +463,46 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
 // instruction slot in sixteen of the wave that sets the pace) disappears from the loop.
 // STAGED (unmasked tiles, block size a compile-time constant up to a tile): the tile's keys go to the lane's row of the LDS key buffer, `staged_row`
 // pointing at the tile's first key there; a loader wave writes the rows out (drain_keys).
-template <int CHUNK, bool MASKED, int BS, bool STAGED = false>
-__device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_t &h, int64_t t0, int64_t my_ntok,
+template <int CHUNK, bool MASKED, int BS, bool STAGED = false, bool RAW = false>
+__device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kRowVecs], uint64_t &h, int64_t t0, int64_t my_ntok,
                                          int32_t &since_key, int32_t block_size, int64_t *__restrict__ keys,
                                          int64_t &key_pos, uint64_t *staged_row = nullptr) {
+    constexpr int TOK = tile_tokens(RAW);  // steps per tile
     static_assert(!STAGED || (!MASKED && BS >= 1 && BS <= 2 * kTT), "keys are staged for whole tiles of blocks up to two tiles");
-    static_assert(BS == 0 || (BS % CHUNK == 0 && (kTT % BS == 0 || BS % kTT == 0)), "block size fits the tiling");
+    static_assert(BS == 0 || (BS % CHUNK == 0 && (TOK % BS == 0 || BS % TOK == 0)), "block size fits the tiling");
     // tokens of this lane that are hashed and lie in this tile or before its end: a block that ends at position p of
     // the tile belongs to the lane iff p <= left (my_ntok is a multiple of the block size)
     const int64_t left64 = my_ntok - t0;
-    const int32_t left = MASKED ? static_cast<int32_t>(left64 < kTT ? (left64 > 0 ? left64 : 0) : kTT) : kTT;
+    const int32_t left = MASKED ? static_cast<int32_t>(left64 < TOK ? (left64 > 0 ? left64 : 0) : TOK) : TOK;
+    // raw tiles: four 4-byte tokens per 16-byte piece; sign-extension + C is one v_mad_i64_i32 off the chain, issued
+    // KVCM_HASH_RAW_AHEAD steps before the step that consumes it
+    const auto raw_token = [&](int s) -> uint32_t {
+        const uint64_t pair = (s & 2) ? a[s / 4].y : a[s / 4].x;
+        return static_cast<uint32_t>((s & 1) ? pair >> 32 : pair);
+    };
+    constexpr int kAhead = KVCM_HASH_RAW_AHEAD;
+    uint64_t pre[kAhead > 0 ? kAhead : 1];
+    if (RAW) {
 #pragma unroll
-    for (int c = 0; c < kTT; c += CHUNK) {
+        for (int i = 0; i < kAhead; ++i) {
+            pre[i] = pre_add_i32(raw_token(i));
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < TOK; c += CHUNK) {
 #pragma unroll
         for (int s = c; s < c + CHUNK; ++s) {
-            h = chain_step(h, (s & 1) ? a[s / 2].y : a[s / 2].x);
+            if (RAW && kAhead > 0) {
+                const uint64_t now = pre[s % kAhead];
+                if (s + kAhead < TOK) {
+                    pre[s % kAhead] = pre_add_i32(raw_token(s + kAhead));
+                }
+                h = chain_step(h, now);
+            } else if (RAW) {
+                h = chain_step(h, pre_add_i32(raw_token(s)));
+            } else {
+                h = chain_step(h, (s & 1) ? a[s / 2].y : a[s / 2].x);
+            }
         }
         bool key_due;
         if (BS == 0) {
@@ -451,14 +511,14 @@ __device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_
             if (key_due) {
                 since_key = 0;
             }
-        } else if (BS <= kTT) {
+        } else if (BS <= TOK) {
             key_due = (c + CHUNK) % BS == 0;  // tiles start on block boundaries
         } else {
-            key_due = c + CHUNK == kTT && (t0 + kTT) % BS == 0;
+            key_due = c + CHUNK == TOK && (t0 + TOK) % BS == 0;
         }
         if (key_due) {
             if (STAGED) {
-                staged_row[BS > kTT ? 0 : (c + CHUNK) / (BS > 0 ? BS : 1) - 1] = h;
+                staged_row[BS > TOK ? 0 : (c + CHUNK) / (BS > 0 ? BS : 1) - 1] = h;
             } else if (!MASKED || c + CHUNK <= left) {
                 keys[key_pos] = static_cast<int64_t>(h);
             }
@@ -467,10 +527,10 @@ __device__ __forceinline__ void run_tile(const ulonglong2 (&a)[kTT / 2], uint64_
     }
 }
 
-__device__ __forceinline__ void read_row(ulonglong2 (&a)[kTT / 2], const uint64_t *row_ptr) {
+__device__ __forceinline__ void read_row(ulonglong2 (&a)[kRowVecs], const uint64_t *row_ptr) {
     const ulonglong2 *row = reinterpret_cast<const ulonglong2 *>(row_ptr);
 #pragma unroll
-    for (int i = 0; i < kTT / 2; ++i) {
+    for (int i = 0; i < kRowVecs; ++i) {
         a[i] = row[i];
     }
 }
@@ -481,7 +541,7 @@ __device__ __forceinline__ void read_row(ulonglong2 (&a)[kTT / 2], const uint64_
 // is bound by memory and not by the chain): the chain wave writes its keys into an LDS buffer instead of to memory, and
 // after every group of tiles in which every request is whole the loader waves write the group out as rows of 512
 // bytes, spread over the next group's tiles (block size 16) or at once.
-template <typename TokT, int CHUNK, int BS, int KS = kKeysDirect>
+template <typename TokT, int CHUNK, int BS, int KS = kKeysDirect, bool RAW = false>
 __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__restrict__ tokens,
                                                               const int64_t *__restrict__ token_offsets, int32_t R,
                                                               int32_t block_size, uint64_t seed,
@@ -493,8 +553,10 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     __shared__ int64_t s_ntok[kReqs];
     static_assert(!KS || (BS >= 1 && BS <= 2 * kTT), "keys are staged for block sizes up to two tiles");
     static_assert(KS != kKeysSpread || BS == 16, "the spread form exists for 16-token blocks");
-    constexpr int G = key_group_tiles(BS);  // tiles per group of staged keys
-    constexpr int kDiv = BS > 0 ? BS : 1;  // the first key of tile t of a group lies at position t * kTT / BS of the row
+    constexpr int TOK = tile_tokens(RAW);        // tokens per request per tile
+    constexpr int G = key_group_tiles(BS, TOK);  // tiles per group of staged keys
+    static_assert(!KS || G >= 1, "a group of staged keys is at least one tile");
+    constexpr int kDiv = BS > 0 ? BS : 1;  // the first key of tile t of a group lies at position t * TOK / BS of the row
     __shared__ __attribute__((aligned(16))) uint64_t s_keys[KS ? 2 * kReqs * kKeyRow : 2];
     __shared__ int64_t s_keypos[KS ? kReqs : 1];
 
@@ -539,8 +601,8 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
     // lane has run out): max and min over the 64 lanes of per-lane tile counts, which fit 32 bits (a request of 2^37
     // tokens does not fit the memory of the device). Rows past R in the last workgroup count for neither.
     const int64_t lane_ntok = s_ntok[lane];
-    const uint32_t ntiles_u = wave_max_u32(static_cast<uint32_t>((lane_ntok + kTT - 1) / kTT));
-    const uint32_t full_u = wave_min_u32(r < R ? static_cast<uint32_t>(lane_ntok / kTT) : 0xFFFFFFFFu);
+    const uint32_t ntiles_u = wave_max_u32(static_cast<uint32_t>((lane_ntok + TOK - 1) / TOK));
+    const uint32_t full_u = wave_min_u32(r < R ? static_cast<uint32_t>(lane_ntok / TOK) : 0xFFFFFFFFu);
     const int64_t ntiles = ntiles_u;  // uniform over the workgroup
     if (ntiles == 0) {
         return;
@@ -553,9 +615,9 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         // ---------------------------------------------------------------- loader waves
         const KeyDrain kd{s_keys, s_keypos, keys, n_stageable};
         if (buffer_loads) {
-            run_loader<BufferLoader<TokT>, TokT, KS, G>(ctx, s_tile, wave - 1, ntiles, lane, kd);
+            run_loader<BufferLoader<TokT, RAW>, TokT, KS, G, TOK>(ctx, s_tile, wave - 1, ntiles, lane, kd);
         } else {
-            run_loader<GlobalLoader<TokT>, TokT, KS, G>(ctx, s_tile, wave - 1, ntiles, lane, kd);
+            run_loader<GlobalLoader<TokT, RAW>, TokT, KS, G, TOK>(ctx, s_tile, wave - 1, ntiles, lane, kd);
         }
         return;
     }
@@ -570,7 +632,7 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         // usable when R is not a multiple of 64.
         return;
     }
-    ulonglong2 cur[kTT / 2], nxt[kTT / 2];
+    ulonglong2 cur[kRowVecs], nxt[kRowVecs];
     read_row(cur, &s_tile[0][lane][0]);
     lds_barrier();  // tile 0 is in registers: its slot may take tile 2
     // Loop control in 32-bit scalars (there are no ordered 64-bit scalar compares, and every vector compare is an issue
@@ -586,15 +648,15 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         // a group of G tiles is staged when all of its tiles are whole for every request
         const int32_t group = k / G;
         const bool staged = KS && (group + 1) * G <= n_stageable;
-        uint64_t *staged_row = KS ? s_keys + ((group & 1) * kReqs + lane) * kKeyRow + (k & (G - 1)) * kTT / kDiv : nullptr;
+        uint64_t *staged_row = KS ? s_keys + ((group & 1) * kReqs + lane) * kKeyRow + (k & (G - 1)) * TOK / kDiv : nullptr;
         if (KS && staged) {
-            run_tile<CHUNK, false, BS, KS != kKeysDirect>(cur, h, static_cast<int64_t>(k) * kTT, my_ntok, since_key, block_size, keys,
+            run_tile<CHUNK, false, BS, KS != kKeysDirect, RAW>(cur, h, static_cast<int64_t>(k) * TOK, my_ntok, since_key, block_size, keys,
                                            key_pos, staged_row);
         } else if (k < n_full) {
-            run_tile<CHUNK, false, BS>(cur, h, static_cast<int64_t>(k) * kTT, my_ntok, since_key, block_size, keys,
+            run_tile<CHUNK, false, BS, false, RAW>(cur, h, static_cast<int64_t>(k) * TOK, my_ntok, since_key, block_size, keys,
                                        key_pos);
         } else {
-            run_tile<CHUNK, true, BS>(cur, h, static_cast<int64_t>(k) * kTT, my_ntok, since_key, block_size, keys,
+            run_tile<CHUNK, true, BS, false, RAW>(cur, h, static_cast<int64_t>(k) * TOK, my_ntok, since_key, block_size, keys,
                                       key_pos);
         }
         lds_barrier();
@@ -608,15 +670,15 @@ __global__ __launch_bounds__(kThreads) void hash_tokens_kernel(const TokT *__res
         const int32_t group1 = (k + 1) / G;  // the same group unless a group is one tile
         const bool staged1 = KS && (group1 + 1) * G <= n_stageable;
         uint64_t *staged_row1 =
-            KS ? s_keys + ((group1 & 1) * kReqs + lane) * kKeyRow + ((k + 1) & (G - 1)) * kTT / kDiv : nullptr;
+            KS ? s_keys + ((group1 & 1) * kReqs + lane) * kKeyRow + ((k + 1) & (G - 1)) * TOK / kDiv : nullptr;
         if (KS && staged1) {
-            run_tile<CHUNK, false, BS, KS != kKeysDirect>(nxt, h, static_cast<int64_t>(k + 1) * kTT, my_ntok, since_key, block_size,
+            run_tile<CHUNK, false, BS, KS != kKeysDirect, RAW>(nxt, h, static_cast<int64_t>(k + 1) * TOK, my_ntok, since_key, block_size,
                                            keys, key_pos, staged_row1);
         } else if (k + 1 < n_full) {
-            run_tile<CHUNK, false, BS>(nxt, h, static_cast<int64_t>(k + 1) * kTT, my_ntok, since_key, block_size, keys,
+            run_tile<CHUNK, false, BS, false, RAW>(nxt, h, static_cast<int64_t>(k + 1) * TOK, my_ntok, since_key, block_size, keys,
                                        key_pos);
         } else {
-            run_tile<CHUNK, true, BS>(nxt, h, static_cast<int64_t>(k + 1) * kTT, my_ntok, since_key, block_size, keys,
+            run_tile<CHUNK, true, BS, false, RAW>(nxt, h, static_cast<int64_t>(k + 1) * TOK, my_ntok, since_key, block_size, keys,
                                       key_pos);
         }
         lds_barrier();
@@ -825,37 +887,66 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
 #define KVCM_LAUNCH_HASH_STAGED(CHUNK, BS, KS)                                                                       \
     hipLaunchKernelGGL((hash_tokens_kernel<TokT, CHUNK, BS, KS>), grid, dim3(kThreads), 0, stream, d_tokens,        \
                        d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
-    if (spread) {
+    // 4-byte tokens from as many requests as take the burst form: tiles of 128 raw tokens (512-byte pieces of the
+    // token stream per request and load instruction instead of 256-byte ones). Cold timings, 16-token blocks, requests
+    // of 4096 tokens, 64-token tiles of pre-added terms / raw tiles: 64 requests 56.8 / 57.3 us, 8192 58.1 / 60.2,
+    // 12 288 66.6 / 62.2, 16 384 77.3 / 66.4, 32 768 149 / 127.
+    const bool raw = !k8 && burst && (block_size == 8 || block_size == 16 || block_size == 32 || block_size == 64 ||
+                                      block_size == 128);
+#define KVCM_LAUNCH_HASH_RAW(BS)                                                                                      \
+    hipLaunchKernelGGL((hash_tokens_kernel<TokT, 8, BS, kKeysBurst, true>), grid, dim3(kThreads), 0, stream, d_tokens, \
+                       d_token_offsets, R, block_size, static_cast<uint64_t>(seed), d_keys, d_key_offsets, force_global)
+    if (raw) {
+        if constexpr (!k8) {
+            switch (block_size) {
+                case 8: KVCM_LAUNCH_HASH_RAW(8); break;
+                case 16: KVCM_LAUNCH_HASH_RAW(16); break;
+                case 32: KVCM_LAUNCH_HASH_RAW(32); break;
+                case 64: KVCM_LAUNCH_HASH_RAW(64); break;
+                default: KVCM_LAUNCH_HASH_RAW(128); break;
+            }
+        }
+    } else if (spread) {
         if constexpr (k8) {
             KVCM_LAUNCH_HASH_STAGED(8, 16, kKeysSpread);
         }
     } else if (block_size == 16) {  // the engines' usual block sizes get kernels of their own
-        if (burst) {
-            KVCM_LAUNCH_HASH_STAGED(8, 16, kKeysBurst);
+        if (k8 && burst) {  // 4-byte tokens take the burst form with raw tiles, above
+            if constexpr (k8) {
+                KVCM_LAUNCH_HASH_STAGED(8, 16, kKeysBurst);
+            }
         } else {
             KVCM_LAUNCH_HASH(8, 16);
         }
     } else if (block_size == 8) {
-        if (burst) {
-            KVCM_LAUNCH_HASH_STAGED(8, 8, kKeysBurst);
+        if (k8 && burst) {  // 4-byte tokens take the burst form with raw tiles, above
+            if constexpr (k8) {
+                KVCM_LAUNCH_HASH_STAGED(8, 8, kKeysBurst);
+            }
         } else {
             KVCM_LAUNCH_HASH(8, 8);
         }
     } else if (block_size == 32) {
-        if (burst) {
-            KVCM_LAUNCH_HASH_STAGED(8, 32, kKeysBurst);
+        if (k8 && burst) {  // 4-byte tokens take the burst form with raw tiles, above
+            if constexpr (k8) {
+                KVCM_LAUNCH_HASH_STAGED(8, 32, kKeysBurst);
+            }
         } else {
             KVCM_LAUNCH_HASH(8, 32);
         }
     } else if (block_size == 64) {
-        if (burst) {
-            KVCM_LAUNCH_HASH_STAGED(8, 64, kKeysBurst);
+        if (k8 && burst) {  // 4-byte tokens take the burst form with raw tiles, above
+            if constexpr (k8) {
+                KVCM_LAUNCH_HASH_STAGED(8, 64, kKeysBurst);
+            }
         } else {
             KVCM_LAUNCH_HASH(8, 64);
         }
     } else if (block_size == 128) {
-        if (burst) {
-            KVCM_LAUNCH_HASH_STAGED(8, 128, kKeysBurst);
+        if (k8 && burst) {  // 4-byte tokens take the burst form with raw tiles, above
+            if constexpr (k8) {
+                KVCM_LAUNCH_HASH_STAGED(8, 128, kKeysBurst);
+            }
         } else {
             KVCM_LAUNCH_HASH(8, 128);
         }
@@ -870,6 +961,7 @@ int32_t launch_hash(const TokT *d_tokens, const int64_t *d_token_offsets, int32_
     } else {
         KVCM_LAUNCH_HASH(1, 0);
     }
+#undef KVCM_LAUNCH_HASH_RAW
 #undef KVCM_LAUNCH_HASH_STAGED
 #undef KVCM_LAUNCH_HASH
     return launch_status();

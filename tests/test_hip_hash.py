@@ -270,3 +270,37 @@ def test_staged_keys_at_other_block_sizes(oracle, bs, dtype):
     got = host(got, np.int64)
     assert (got[:len(want)] == want).all()
     assert (got[len(want):] == -7).all()
+
+
+@pytest.mark.parametrize("general_loader", [False, True])
+@pytest.mark.parametrize("bs", [8, 16, 32, 64, 128])
+def test_raw_tiles_of_4_byte_tokens(oracle, force_general_hash_loader, bs, general_loader):
+    """Launches of 12 288 requests or more of 4-byte tokens use tiles of 128 RAW tokens per request (the chain wave
+    sign-extends and adds the constant itself) and write their keys as whole rows. Request lengths sit on and around
+    the tile width (64, 127, 128, 129, 192, 256, ...), on multiples of a key group, and in between; every workgroup
+    mixes them; tokens cover the whole signed 32-bit range. Both loaders. Exact against the oracle."""
+    force_general_hash_loader(general_loader)
+    rng = np.random.default_rng(41 + bs)
+    R = 12288 + 77                                   # the last workgroup is partial
+    group = 64 * bs                                  # tokens that yield one group of staged keys
+    menu = np.array([0, 1, bs - 1, bs, 63, 64, 65, 127, 128, 129, 191, 192, 193, 255, 256, 257, 384, 511, 512,
+                     group - 1, group, group + 1, group + 128, group + 129, 2 * group, 2 * group + 64 + bs])
+    lens = menu[rng.integers(0, len(menu), size=R)].astype(np.int64)
+    lens[rng.random(R) < 0.3] = rng.integers(0, 2 * group + 300)      # and anything in between
+    lens[:64] = 2 * group + 128                      # one workgroup of equal, whole requests: every group staged
+    lens[64:128] = np.where(np.arange(64) % 2 == 0, group + 128, 2 * group)
+    scale = max(1, int(lens.sum() // 40_000_000) + 1)                 # keep the launch under ~160 MB of tokens
+    if scale > 1:
+        lens[128:] = lens[128:] // scale
+    toff = np.zeros(R + 1, dtype=np.int64)
+    np.cumsum(lens, out=toff[1:])
+    flat = rng.integers(-2**31, 2**31, size=int(toff[-1]), dtype=np.int64).astype(np.int32)
+    flat[:16] = [-2**31, 2**31 - 1, -1, 0, 1, -2, 2**31 - 2, -2**31 + 1] * 2
+    print(f"raw tiles: bs={bs} general_loader={general_loader} R={R} tokens={int(toff[-1])}", flush=True)
+    want, woff = oracle.hash_tokens(flat, bs, token_offsets=toff, seed=-3)
+    keys = torch.full((len(want) + 64,), -7, dtype=torch.int64, device="cuda")
+    got, off = _h().hash_tokens(dev(flat), bs, token_offsets=dev(toff), seed=-3, keys=keys, key_offsets=dev(woff))
+    sync()
+    got = host(got, np.int64)
+    assert (got[:len(want)] == want).all()
+    assert (got[len(want):] == -7).all()
