@@ -32,9 +32,6 @@ namespace {
 #ifndef KVCM_HASH_RAW_AHEAD
 #define KVCM_HASH_RAW_AHEAD 1
 #endif
-#ifndef KVCM_HASH_BURST_ISSUE_WHOLE
-#define KVCM_HASH_BURST_ISSUE_WHOLE 1
-#endif
 #ifndef KVCM_HASH_DRAIN_POLICY
 #define KVCM_HASH_DRAIN_POLICY 0
 #endif
@@ -422,8 +419,11 @@ __device__ __forceinline__ void run_loader(const LoaderCtx<TokT> &ctx, uint64_t 
         // instructions sits in the CU's memory pipeline in front of the chain wave's key stores
         // (which of the two forms runs is a compile-time matter: with both in one loop body the compiler waits for
         // all outstanding loads where the paths meet, and a kernel that does so takes 80 us for a batch instead of 58)
-        if (KS == kKeysSpread || (KS == kKeysBurst && KVCM_HASH_BURST_ISSUE_WHOLE && sizeof(TokT) == 8)) {
-            // no key stores of the chain wave to keep out of the way of: 2 to 5 % faster from 4096 requests than in halves
+        if (KS == kKeysSpread || (KS == kKeysBurst && sizeof(TokT) == 8)) {
+            // no key stores of the chain wave to keep out of the way of: 2 to 5 % faster from 4096 requests than in
+            // halves (spread form); in the burst form of 8-byte tokens 4 % at 10 240 and 12 288 requests, 7 to 10 % for
+            // the prefix chain up to 2048 chains, nothing at 16 384. Raw tiles of 4-byte tokens lose 5 % by it at
+            // 16 384 requests (66.8 against 63.6 us) and keep the halves.
             if (mine && nxt + kLoaders < nt) {
                 ld.issue(static_cast<int64_t>(nxt + kLoaders) * TOK);
             }
