@@ -149,3 +149,35 @@ def test_a_block_of_more_runs_than_an_argument_block_holds_is_uploaded(oracle):
     bgs.batch_gather_kv_caches(table, st, tidx.reshape(-1).tolist(), list(range(B)), T, D)
     sync()
     assert (host(st, np.uint16) == want).all()
+
+
+def test_host_list_call_can_be_captured_and_replayed(oracle):
+    """The host-list entry points launch kernels and nothing else (no upload, no allocation, no memset): a captured
+    call carries its index tables inside the graph. Replayed three times with other pool contents each time, with eager
+    work and synchronisations in between, every replay against the oracle."""
+    bgs = _ops()
+    P, T, D, B, n_slots = 4, 16, 256, 100, 4096
+    rng = np.random.default_rng(21)
+    tidx = rng.permutation(n_slots)[:B * T].reshape(B, T).astype(np.int32)   # unrelated slots: three launches per call
+    lst, slots = tidx.reshape(-1).tolist(), list(range(B))
+    pool = torch.zeros((P, n_slots, D), dtype=torch.int16, device="cuda")
+    table = ptr_table([pool[p] for p in range(P)])
+    st = torch.zeros((B, P, T, D), dtype=torch.int16, device="cuda")
+    bgs.batch_gather_kv_caches(table, st, lst, slots, T, D)  # eager once: the library and its kernels are loaded
+    sync()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.graph(graph, stream=side):
+        bgs.batch_gather_kv_caches(table, st, lst, slots, T, D, pool_token_slots=n_slots)
+    lst[:] = [0] * len(lst)  # the lists are the caller's again: the graph must not look at them
+    for rep in range(3):
+        pools = cases.pool_u16(P, n_slots, D, seed=100 + rep)
+        pool.copy_(torch.stack([dev(p) for p in pools]))
+        st.fill_(-1)
+        sync()
+        graph.replay()
+        sync()
+        want = np.zeros((B, P, T, D), dtype=np.uint16)
+        oracle.batch_gather(pools, want, tidx, None, T, D * 2)
+        assert (host(st, np.uint16) == want).all(), rep
