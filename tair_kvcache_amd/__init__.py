@@ -13,4 +13,4 @@ Operators (same names and argument order as the reference's Python operator modu
 All device work goes through libkvcm_hip.so (include/kvcm_hip.h); there is no CPU fallback.
 """
 
-__version__ = "0.1.0"
+__version__ = "0.2.0"

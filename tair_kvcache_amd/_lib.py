@@ -94,6 +94,11 @@ def lib():
                     raise KvcmLibraryError(
                         f"{LIB_PATH} is not built; run `python -m tair_kvcache_amd.build` (needs hipcc). "
                         "There is no CPU fallback.")
+                # torch first: it brings its own copy of the HIP runtime, and a process must end up with ONE runtime.
+                # Loaded after torch, this library binds to the runtime torch has already loaded; loaded before it,
+                # the library pulls in the system's copy, torch then loads its own, and the kernels registered with
+                # one runtime are launched on streams of the other ("no ROCm-capable device is detected").
+                import torch  # noqa: F401
                 try:
                     L = C.CDLL(LIB_PATH)
                 except OSError as e:
