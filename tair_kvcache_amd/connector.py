@@ -237,6 +237,7 @@ class DataTransferManager:
         self._stream_lock = threading.Lock()
         self._streams: Dict[str, Any] = {}
         self._slot_buffer_cache: Dict[int, Any] = {}
+        self._tls = threading.local()
 
     def _stream(self, which: str):
         s = self._streams.get(which)
@@ -256,6 +257,14 @@ class DataTransferManager:
     @property
     def _load_stream(self):
         return self._stream("load")
+
+    def _thread_event(self):
+        """The event a worker thread waits for its copy with: one per thread, recorded anew for every task (a thread
+        has one task at a time)."""
+        ev = getattr(self._tls, "event", None)
+        if ev is None:
+            ev = self._tls.event = torch.cuda.Event(blocking=_EVENT_BLOCKING)
+        return ev
 
     def submit_task(self, func, *args, **kwargs):
         return self._io_executor.submit(func, *args, **kwargs)
@@ -298,14 +307,17 @@ class DataTransferManager:
         try:
             result = self._transfer_client.LoadKvCaches(remote_uris, self._slot_buffers(slots))
             if result == ok:
-                with torch.cuda.stream(self._load_stream):
-                    batch_gather_scatter_helper.batch_scatter_kv_caches(
-                        self._kvcache_info.all_kvcache_ptr_tensor_gpu, self._copy_buffer_allocator._raw_buffer,
-                        self._flat_indices(block_token_indices), slots, self._manager_block_size,
-                        self._kvcache_info.per_token_per_layer_dim_size,
-                        pool_token_slots=self._kvcache_info.local_token_num)
-                    done = torch.cuda.Event(blocking=_EVENT_BLOCKING)
-                    done.record(self._load_stream)
+                # launched on the load stream by handing the stream over, not by making it torch's current one:
+                # entering a stream context and building an event object are interpreter time, which the worker
+                # threads serialise
+                stream = self._load_stream
+                batch_gather_scatter_helper.batch_scatter_kv_caches(
+                    self._kvcache_info.all_kvcache_ptr_tensor_gpu, self._copy_buffer_allocator._raw_buffer,
+                    self._flat_indices(block_token_indices), slots, self._manager_block_size,
+                    self._kvcache_info.per_token_per_layer_dim_size,
+                    pool_token_slots=self._kvcache_info.local_token_num, stream=stream)
+                done = self._thread_event()
+                done.record(stream)
                 done.synchronize()
         finally:
             self._copy_buffer_allocator.free_buffer(slots)
@@ -353,17 +365,17 @@ class DataTransferManager:
                   kvcache_ready_event: Optional[torch.cuda.Event] = None):
         slots = None
         try:
-            with torch.cuda.stream(self._save_stream):
-                if kvcache_ready_event is not None:
-                    kvcache_ready_event.wait()
-                slots = self._copy_buffer_allocator.alloc_buffer_idx_blocking(len(remote_uris))
-                batch_gather_scatter_helper.batch_gather_kv_caches(
-                    self._kvcache_info.all_kvcache_ptr_tensor_gpu, self._copy_buffer_allocator._raw_buffer,
-                    self._flat_indices(block_token_indices), slots, self._manager_block_size,
-                    self._kvcache_info.per_token_per_layer_dim_size,
-                    pool_token_slots=self._kvcache_info.local_token_num)
-                done = torch.cuda.Event(blocking=_EVENT_BLOCKING)
-                done.record(self._save_stream)
+            stream = self._save_stream
+            if kvcache_ready_event is not None:
+                kvcache_ready_event.wait(stream)
+            slots = self._copy_buffer_allocator.alloc_buffer_idx_blocking(len(remote_uris))
+            batch_gather_scatter_helper.batch_gather_kv_caches(
+                self._kvcache_info.all_kvcache_ptr_tensor_gpu, self._copy_buffer_allocator._raw_buffer,
+                self._flat_indices(block_token_indices), slots, self._manager_block_size,
+                self._kvcache_info.per_token_per_layer_dim_size,
+                pool_token_slots=self._kvcache_info.local_token_num, stream=stream)
+            done = self._thread_event()
+            done.record(stream)
             done.synchronize()
             if isinstance(block_token_indices, torch.Tensor) and block_token_indices.is_cuda and \
                     blocks_idx_error(block_token_indices.device):

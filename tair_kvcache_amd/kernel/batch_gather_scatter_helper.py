@@ -109,8 +109,15 @@ def _host_i32(values, name):
     return values.buffer_info()[0], len(values), values
 
 
+def _stream(stream, device):
+    """`stream` of a call: None = the current torch stream of `device`, else a torch.cuda.Stream or a raw handle."""
+    if stream is None:
+        return stream_handle(device)
+    return getattr(stream, "cuda_stream", stream)
+
+
 def _run(host_fn, device_fn, kv_caches_ptrs_tensor, staging, block_token_indices, block_indices,
-         num_tokens_per_block, dim_size_per_token_per_layer, sm_count, pool_token_slots):
+         num_tokens_per_block, dim_size_per_token_per_layer, sm_count, pool_token_slots, stream=None):
     """Host index lists take the entry point that carries them in the kernel's argument block; anything on the GPU
     (or a block of more runs than an argument block holds) takes the device-index entry point."""
     tok = _host_i32(block_token_indices, "block_token_indices")
@@ -122,18 +129,25 @@ def _run(host_fn, device_fn, kv_caches_ptrs_tensor, staging, block_token_indices
         if tok[1] != B * T:
             raise ValueError(f"block_token_indices has {tok[1]} entries, expected {B} blocks x {T}")
         rc = host_fn(ptr(kv_caches_ptrs_tensor), P, ptr(staging), block_bytes, slots, tok[0], sl[0], B, T, row_bytes,
-                     int(pool_token_slots or 0), _cap(sm_count), stream_handle(device))
+                     int(pool_token_slots or 0), _cap(sm_count), _stream(stream, device))
         if rc == _lib.ERR_OUT_OF_RANGE:
             raise ValueError(f"index out of range: staging slots must lie in [0, {slots}), token slots below "
                              f"pool_token_slots ({pool_token_slots})")
         if rc != _lib.ERR_TOO_LARGE:
             _lib.check(rc, host_fn.__name__)
             return
-    device, P, T, row_bytes, block_bytes, tidx, sidx, B = _prepare(
-        kv_caches_ptrs_tensor, staging, block_token_indices, block_indices, num_tokens_per_block,
-        dim_size_per_token_per_layer)
+    if hasattr(stream, "cuda_stream"):
+        # list arguments are uploaded on torch's current stream: that has to be the stream of the launch
+        with torch.cuda.stream(stream):
+            device, P, T, row_bytes, block_bytes, tidx, sidx, B = _prepare(
+                kv_caches_ptrs_tensor, staging, block_token_indices, block_indices, num_tokens_per_block,
+                dim_size_per_token_per_layer)
+    else:
+        device, P, T, row_bytes, block_bytes, tidx, sidx, B = _prepare(
+            kv_caches_ptrs_tensor, staging, block_token_indices, block_indices, num_tokens_per_block,
+            dim_size_per_token_per_layer)
     rc = device_fn(ptr(kv_caches_ptrs_tensor), P, ptr(staging), block_bytes, ptr(tidx), ptr(sidx), B, T, row_bytes,
-                   _cap(sm_count), stream_handle(device))
+                   _cap(sm_count), _stream(stream, device))
     _lib.check(rc, device_fn.__name__)
 
 
@@ -149,12 +163,13 @@ def batch_gather_kv_caches(
         num_tokens_per_block: int,
         dim_size_per_token_per_layer: int,
         sm_count: int = 3,
-        *, pool_token_slots: int = 0):
-    """dst[sb[b], p, t, :] = pool_p[idx[b*T + t], :]  (batch_gather_scatter_helper.py:49-98)."""
+        *, pool_token_slots: int = 0, stream=None):
+    """dst[sb[b], p, t, :] = pool_p[idx[b*T + t], :]  (batch_gather_scatter_helper.py:49-98).
+    `stream` (keyword only): a torch.cuda.Stream to launch on instead of torch's current one."""
     L = lib()
     _run(L.kvcm_hip_batch_gather_host_idx, L.kvcm_hip_batch_gather, kv_caches_ptrs_tensor, dst_tensor,
          block_token_indices, dst_block_indices, num_tokens_per_block, dim_size_per_token_per_layer, sm_count,
-         pool_token_slots)
+         pool_token_slots, stream)
 
 
 def batch_scatter_kv_caches(
@@ -165,14 +180,14 @@ def batch_scatter_kv_caches(
         num_tokens_per_block: int,
         dim_size_per_token_per_layer: int,
         sm_count: int = 3,
-        *, pool_token_slots: int = 0):
+        *, pool_token_slots: int = 0, stream=None):
     """pool_p[idx[b*T + t], :] = src[sb[b], p, t, :]  (batch_gather_scatter_helper.py:155-205).
 
     Two work blocks that name the same pool row race; callers must not pass duplicates."""
     L = lib()
     _run(L.kvcm_hip_batch_scatter_host_idx, L.kvcm_hip_batch_scatter, kv_caches_ptrs_tensor, src_tensor,
          block_token_indices, src_block_indices, num_tokens_per_block, dim_size_per_token_per_layer, sm_count,
-         pool_token_slots)
+         pool_token_slots, stream)
 
 
 def paged_gather_kv_caches(kv_caches_ptrs_tensor, dst_tensor, run_start_slots: IndexArg,

@@ -181,3 +181,38 @@ def test_host_list_call_can_be_captured_and_replayed(oracle):
         want = np.zeros((B, P, T, D), dtype=np.uint16)
         oracle.batch_gather(pools, want, tidx, None, T, D * 2)
         assert (host(st, np.uint16) == want).all(), rep
+
+
+@pytest.mark.parametrize("form", ["lists", "device_tensors", "list_and_tensor"])
+def test_stream_argument_launches_on_that_stream(oracle, form):
+    """`stream=` hands the launch a stream of the caller's instead of torch's current one (what DataTransferManager's
+    worker threads do): the copy is ordered behind work queued on that stream before it, whichever way the indices
+    arrive -- host lists, device tensors, or a list that has to be uploaded on that stream first."""
+    bgs = _ops()
+    P, T, D, B, n_slots = 4, 16, 512, 64, 4096
+    pools = cases.pool_u16(P, n_slots, D)
+    tidx = cases.token_idx_from_blocks(cases.block_table(n_slots // T, B), T)
+    sidx = np.arange(B, dtype=np.int32)
+    want = np.zeros((B, P, T, D), dtype=np.uint16)
+    oracle.batch_gather(pools, want, tidx, sidx, T, D * 2)
+    pool = torch.zeros((P, n_slots, D), dtype=torch.int16, device="cuda")
+    table = ptr_table([pool[p] for p in range(P)])
+    st = torch.zeros((B, P, T, D), dtype=torch.int16, device="cuda")
+    fresh = torch.stack([dev(p) for p in pools])
+    d_tidx, d_sidx = dev(tidx.reshape(-1)), dev(sidx)
+    sync()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        filler = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+        for _ in range(20):
+            filler.add_(1)          # work in front of ...
+        pool.copy_(fresh)           # ... the copy that fills the pool, all on the side stream
+    # torch's current stream is the default one here: only the stream argument orders the gather behind the fill
+    if form == "lists":
+        bgs.batch_gather_kv_caches(table, st, tidx.reshape(-1).tolist(), sidx.tolist(), T, D, stream=side)
+    elif form == "device_tensors":
+        bgs.batch_gather_kv_caches(table, st, d_tidx, d_sidx, T, D, stream=side)
+    else:
+        bgs.batch_gather_kv_caches(table, st, tidx.reshape(-1).tolist(), d_sidx, T, D, stream=side)
+    side.synchronize()
+    assert (host(st, np.uint16) == want).all()
