@@ -17,6 +17,8 @@
 //               tile periods, so HBM latency stays off the chain. In launches of thousands of requests they also
 //               write the keys out: the chain wave leaves them in an LDS buffer, and whole 512-byte rows per
 //               request go to memory (kKeysSpread / kKeysBurst) instead of one 8-byte store per key and lane.
+//               With 4-byte tokens such launches use tiles of 128 RAW tokens (512-byte row segments here too): the
+//               loaders store what they loaded and the chain wave converts, one step ahead of its use.
 // Roofline: HBM for many requests (8*block_size + 8 bytes per key); for few requests the bound is the
 // dependent-instruction latency of the chain wave, which no amount of bandwidth removes.
 #include "kvcm_internal.h"
@@ -832,7 +834,9 @@ constexpr int32_t kForceGeneralLoader = KVCM_TEST_FORCE_GENERAL_LOADER;
 //                   16 384: 85 / 81 / 78  32 768: 159 / 151 / 151
 // 8-byte tokens: direct below 2048 requests (there the spread form gains 2 to 4 % on tokens from HBM and loses as much
 // on resident ones, and costs requests of 1024 tokens 6 %), spread from 2048, burst from 10 240.
-// 4-byte tokens: direct below 12 288, burst from there (the spread form would gain 3 % between 10 240 and 16 384
+// 4-byte tokens: direct below 12 288, burst from there -- and the burst form of 4-byte tokens is the one with raw tiles
+// (RAW = true; the 4-byte figures of these tables are those of the 64-token tiles of pre-added terms it replaced:
+// 16 384 requests 78 -> 62-66 us) (the spread form would gain 3 % between 10 240 and 16 384
 // requests: not worth one more kernel).
 // Other block sizes, direct / burst:
 //   block size 1, 8-byte tokens   64: 146 / 129   2048: 158 / 136   8192: 241 / 161   16 384: 300 / 202   32 768: 641 / 415
