@@ -23,9 +23,9 @@ from .. import _lib
 from .._torch_util import as_device_i32, lib, ptr, require_cuda, stream_handle
 
 try:  # one C loop over a list (flat or nested); absent only when the package was not built with its build.py
-    from .._kvcm_pylist import pack_i32 as _pack_i32
+    from .._kvcm_pylist import blocks_idx as _blocks_idx_c, pack_i32 as _pack_i32
 except ImportError:  # host-side convenience only: the lists then go through array('i'), three times slower
-    _pack_i32 = None
+    _pack_i32 = _blocks_idx_c = None
 
 IndexArg = Union[List[int], Sequence[int], torch.Tensor]
 
@@ -100,6 +100,9 @@ def _host_i32(values, name):
         if t.dtype != torch.int32 or not t.is_contiguous():
             t = t.to(torch.int32).contiguous()
         return t.data_ptr(), t.numel(), t
+    packed = getattr(values, "packed_int32", None)  # a HostBlockIndex of tair_kvcache_amd.connector
+    if packed is not None:
+        values = packed
     if isinstance(values, bytes):  # already packed by pack_index_list
         return values, len(values) // 4, values
     if not (isinstance(values, array) and values.typecode == "i"):

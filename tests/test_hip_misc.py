@@ -483,3 +483,56 @@ def test_device_built_indices_that_leave_the_block_list_are_not_saved():
         assert (want == ClientErrorCode.ER_OK) == all(u in client.store for u in uris)
     assert connector.blocks_idx_error("cuda") is False  # read and cleared by the task that met it
     mgr.shutdown()
+
+
+def test_host_built_block_index_through_the_transfer_manager(oracle):
+    """generate_blocks_idx_host (the reference's list flow, v1_connector.py:308-320, without the Python double loop)
+    -> slices of it handed to save_task and load_task; manager blocks of 64 tokens over engine blocks of 16. Stored
+    bytes equal the oracle's staging layout and the caches come back byte for byte."""
+    from tair_kvcache_amd import connector
+    from tair_kvcache_amd.client_types import ClientErrorCode
+    from tair_kvcache_amd.kernel.gather_scatter_helper import CopyBufferAllocator
+    L, nblk, T_eng, T_mgr, H, hd = 3, 96, 16, 64, 2, 64
+    rng = np.random.default_rng(5)
+    np_caches = [rng.integers(0, 65536, size=(2, nblk, T_eng, H, hd), dtype=np.uint16) for _ in range(L)]
+    kv = {f"layer{l}": dev(np_caches[l]).view(torch.bfloat16) for l in range(L)}
+    info = connector.register_kv_caches(kv, manager_block_size=T_mgr, local_block_size=T_eng)
+    alloc = CopyBufferAllocator(torch.device("cpu"), torch.bfloat16, list(info.per_manager_block_shape), 16)
+    client = FakeTransferClient()
+    mgr = connector.DataTransferManager(info, T_mgr, alloc, client, max_workers=2)
+    local_block_ids = cases.block_table(nblk, 40).tolist()  # 40 engine blocks = 10 manager blocks
+    manager_blocks = [9, 0, 3, 4, 5, 7]
+    idx = connector.generate_blocks_idx_host(manager_blocks, local_block_ids, T_mgr, T_eng)
+    idx_np, bad = oracle.generate_blocks_idx(np.array(manager_blocks, dtype=np.int32),
+                                             np.array(local_block_ids, dtype=np.int32), T_mgr, T_eng)
+    assert bad == 0 and idx.tolist() == idx_np.tolist()
+    n = len(manager_blocks)
+    print(f"host-built index: {n} manager blocks of {T_mgr} over engine blocks of {T_eng}", flush=True)
+    uris = [f"file:///kv/h?blkid={i}" for i in range(n)]
+    done, results = threading.Event(), []
+    multi = connector.MultiResult(2, lambda r: (results.append(r), done.set()))
+    mgr.submit_task(mgr.save_task, multi, 0, uris[:4], idx[:4], None)
+    mgr.submit_task(mgr.save_task, multi, 1, uris[4:], idx[4:], None)
+    assert done.wait(60)
+    assert results[0] == [[ClientErrorCode.ER_OK] * 4, [ClientErrorCode.ER_OK] * 2]
+    pools = [np_caches[l][kvi].reshape(nblk * T_eng, H * hd) for l in range(L) for kvi in (0, 1)]
+    want = np.zeros((n, 2 * L, T_mgr, H * hd), dtype=np.uint16)
+    oracle.batch_gather(pools, want, idx_np, None, T_mgr, H * hd * 2)
+    for i, uri in enumerate(uris):
+        assert client.store[uri] == want[i].tobytes(), i
+    kv2 = {k: torch.zeros_like(v) for k, v in kv.items()}
+    mgr2 = connector.DataTransferManager(connector.register_kv_caches(kv2, T_mgr, T_eng), T_mgr, alloc, client,
+                                         max_workers=2)
+    done2, res2 = threading.Event(), []
+    mgr2.submit_task(mgr2.load_task, connector.MultiResult(1, lambda r: (res2.append(r), done2.set())), 0, uris, idx)
+    assert done2.wait(60)
+    assert res2[0] == [[ClientErrorCode.ER_OK] * n] and alloc._inuse_count == 0
+    sync()
+    touched = np.unique(idx_np // T_eng)
+    rest = np.setdiff1d(np.arange(nblk), touched)
+    for l in range(L):
+        g = host(kv2[f"layer{l}"].view(torch.int16), np.uint16)
+        assert (g[:, touched] == np_caches[l][:, touched]).all()
+        assert not g[:, rest].any()
+    mgr.shutdown()
+    mgr2.shutdown()

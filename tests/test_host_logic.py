@@ -360,3 +360,50 @@ def test_index_lists_are_packed_in_c_flat_and_nested():
                 bgs.pack_index_list(bad)
     finally:
         bgs._pack_i32 = helper
+
+
+def test_generate_blocks_idx_host_equals_the_reference_loop(oracle):
+    """generate_blocks_idx_host: the values of the reference's Python double loop (v1_connector.py:308-320) and of the
+    oracle, for manager blocks smaller than, equal to and larger than engine blocks; slices by block like the nested
+    list the reference returns; asserts like the reference when a manager block reaches beyond the block list."""
+    import numpy as np
+    from tair_kvcache_amd import connector
+
+    def reference_loop(manager_block_idxes, local_block_ids, T_mgr, T_eng):
+        blocks_idx = []
+        for m in manager_block_idxes:
+            row = []
+            for i in range(T_mgr):
+                tok = m * T_mgr + i
+                assert tok // T_eng < len(local_block_ids)
+                row.append(local_block_ids[tok // T_eng] * T_eng + tok % T_eng)
+            blocks_idx.append(row)
+        return blocks_idx
+
+    rng = np.random.default_rng(3)
+    for T_mgr, T_eng in ((16, 16), (64, 16), (16, 64), (24, 16), (1, 1), (128, 128)):
+        local = rng.permutation(5000)[:300].tolist()
+        n_mgr = len(local) * T_eng // T_mgr
+        mgr = rng.integers(0, n_mgr, size=77).tolist()
+        want = reference_loop(mgr, local, T_mgr, T_eng)
+        got = connector.generate_blocks_idx_host(mgr, local, T_mgr, T_eng)
+        assert len(got) == 77 and got.tolist() == want
+        idx, bad = oracle.generate_blocks_idx(np.array(mgr, dtype=np.int32), np.array(local, dtype=np.int32), T_mgr, T_eng)
+        assert bad == 0 and idx.tolist() == want
+        assert got[10:20].tolist() == want[10:20] and got[5] == want[5] and got[-1] == want[-1]
+        assert len(got[70:200]) == 7 and len(got[80:90]) == 0
+        assert bgs._host_i32(got[3:9], "x")[1] == 6 * T_mgr
+        # tuples, and anything that is not a plain list (the Python loop)
+        assert connector.generate_blocks_idx_host(tuple(mgr), tuple(local), T_mgr, T_eng).tolist() == want
+        assert connector.generate_blocks_idx_host(np.array(mgr), local, T_mgr, T_eng).tolist() == want
+    with pytest.raises(AssertionError):
+        connector.generate_blocks_idx_host([19], list(range(19)), 16, 16)
+    with pytest.raises(AssertionError):
+        connector.generate_blocks_idx_host([-1], list(range(19)), 16, 16)
+    with pytest.raises(ValueError):
+        connector.generate_blocks_idx_host([0], [2 ** 31], 16, 16)
+    with pytest.raises(ValueError):
+        connector.generate_blocks_idx_host([0], [1.5], 16, 16)
+    with pytest.raises(ValueError):
+        connector.generate_blocks_idx_host([0], [2 ** 30], 16, 16)  # the slot itself does not fit 32 bits
+    assert len(connector.generate_blocks_idx_host([], [1, 2], 16, 16)) == 0
