@@ -152,6 +152,58 @@ def hash_figures(torch, hashing, tokens, block, reps):
                   "hash_floor_ms": round(L * HASH_STEP_FLOOR_NS * 1e-6, 4)}
 
 
+def cold_batches_ms(torch, _lib, tokens, token_off, key_off, keys_expected, R, block, n=10, reps=7, sweep_gib=2):
+    """(a) Mean milliseconds per launch of n one-batch launches in a row on n DIFFERENT copies of the batch, none of them
+    read since a pass over `sweep_gib` GiB of other memory, one pair of events around the n launches: every launch reads
+    its tokens from HBM, and no pair of events sits around a single launch. (b) What a pair of events around a single
+    launch adds to that launch's reading: per-launch time with an event after every launch minus the mean without, on
+    the resident batch. The n key arrays must equal keys_expected (the batch's keys, already checked)."""
+    device = tokens.device
+    copies = [tokens.clone() for _ in range(n)]
+    outs = [torch.zeros_like(keys_expected) for _ in range(n)]
+    stream = torch.cuda.current_stream().cuda_stream
+    argsets = [(c.data_ptr(), token_off.data_ptr(), R, block, 0, o.data_ptr(), key_off.data_ptr(), stream)
+               for c, o in zip(copies, outs)]
+
+    def launch(a):
+        rc = _lib.lib().kvcm_hip_hash_tokens(*a)
+        if rc != 0:
+            raise SystemExit(f"bench.py: kvcm_hip_hash_tokens failed with code {rc}")
+
+    sweep = torch.zeros(sweep_gib * 2**30, dtype=torch.uint8, device=device)
+    means = []
+    for _ in range(reps):
+        sweep.add_(1)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for a in argsets:
+            launch(a)
+        e1.record()
+        torch.cuda.synchronize()
+        means.append(e0.elapsed_time(e1) / n)
+    del sweep
+    for o in outs:
+        if not torch.equal(o, keys_expected):
+            raise SystemExit("bench.py: a copy of the batch hashed to other keys than the batch")
+    plain, single = [], []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            launch(argsets[0])
+        e1.record()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+        ev[0].record()
+        for i in range(n):
+            launch(argsets[0])
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        plain.append(e0.elapsed_time(e1) / n)
+        single.append(sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(n))[n // 2])
+    med = lambda v: sorted(v)[len(v) // 2]
+    return med(means), med(single) - med(plain)
+
+
 def cold_ms(torch, fn, device, reps=7, sweep_gib=2):
     """Median milliseconds of one call of fn when every call follows a read-modify-write pass over `sweep_gib` GiB of
     other memory: the 256 MiB memory-side cache and the L2 then hold someone else's dirty lines and the call's inputs
@@ -790,6 +842,7 @@ def main():
     # hand-over from the 8 ms load kernel before it
     ms_hash_b2b = gpu_ms(torch, hash_once, 20)
     ms_hash_cold = cold_ms(torch, hash_once, device)
+    ms_hash_cold_ten, ms_event_pair = cold_batches_ms(torch, _lib, d_tokens, d_token_off, d_key_off, d_keys, REQUESTS, T)
     # ApplyPrefixHash (kv_cache_manager/optimizer/trace_converter/trace_util.cc:47-56) on as many chains: the same
     # 16 384 x 4096 values taken as digests, a key after every step (as many bytes written as read)
     del sat_keys
@@ -878,12 +931,18 @@ def main():
         "keys_per_s_back_to_back": round(d_keys.numel() / (ms_hash_b2b * 1e-3)),
         "hash_ms_back_to_back_before_the_steps": round(ms_hash_b2b_first, 4),
         "hash_ms_cold": round(ms_hash_cold, 4),
+        "hash_ms_cold_ten_batches": round(ms_hash_cold_ten, 4),
+        "event_pair_around_one_launch_us": round(ms_event_pair * 1e3, 2),
         "hash_floor_us": round(TOKENS_PER_REQ * HASH_STEP_FLOOR_NS * 1e-3, 2),
         "hash_note": "one request is a serial chain of 4096 dependent steps, three dependent VALU instructions each at "
                      "3.65 ns: 64 chains cannot finish in less than hash_floor_us; more than 1e9 keys/s needs 256 or more "
                      "chains in flight (keys_per_s_4_batches). hash_ms is the launch inside the step, behind the 8 ms load kernel; "
                      "the back-to-back figures repeat the launch on tokens that then sit in the caches; hash_ms_cold "
-                     "follows a pass over 2 GiB of other memory, which is how a batch that has just arrived is hashed",
+                     "follows a pass over 2 GiB of other memory, which is how a batch that has just arrived is hashed. hash_ms and "
+                     "hash_ms_cold are each one launch between its own pair of events, which reads "
+                     "event_pair_around_one_launch_us more than the launch takes; hash_ms_cold_ten_batches is the mean of "
+                     "ten launches in a row on ten copies of the batch, none read since such a pass, one pair of events "
+                     "around the ten",
         "keys_per_s_4_batches": round(few_keys / (ms_few * 1e-3)), "hash_chains_4_batches": few_R,
         "hash_ms_4_batches": round(ms_few, 4), "hash_ms_4_batches_cold": round(ms_few_cold, 4),
         "keys_per_s_4_batches_cold": round(few_keys / (ms_few_cold * 1e-3)),
