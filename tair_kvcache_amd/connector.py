@@ -139,7 +139,7 @@ def generate_blocks_idx_host(manager_block_idxes: Sequence[int], local_block_ids
     """generate_blocks_idx for callers that hold their block lists as Python lists and hand the result to
     DataTransferManager task by task, as the reference connector does (v1_connector.py:455,499-515): the same values
     as the reference's Python double loop (:308-320), computed in one C loop (2 us for 128 blocks of 16 tokens instead
-    of 181 us) and kept packed, so that every task's slice goes to the host-list gather/scatter entry points as it is
+    of 258 us) and kept packed, so that every task's slice goes to the host-list gather/scatter entry points as it is
     -- no device kernel, no upload, and whole-block tasks take the block-table form of the copy kernel.
     AssertionError when a manager block reaches beyond local_block_ids, like the reference's assert."""
     T_mgr, T_eng = int(manager_block_size), int(local_block_size)
